@@ -1,0 +1,273 @@
+"""The cache: a slot per sequence, keys and values per cache line in pages, and
+per-sequence state of fixed size.
+
+The reference holds one sequence: per layer two planes ``[Hkv, max_seq, D]`` and one
+scalar position (rocml/src/cache.rs:45-138, rocml/src/forward/mod.rs:84); a reset
+only sets the position to zero because rows beyond it are never read
+(rocml/src/forward/mod.rs:224-232), while the fixed-size state of its other
+architecture is zeroed on reset (rocml/src/qwen35/cache/mod.rs:289-298).  Both rules
+are kept here, for many sequences:
+
+* a **slot** stands for one live sequence and knows its length;
+* cache lines (one per execution of a layer that owns a cache) with the same needs form
+  a **group** with storage of its own.  A key/value group is a pool of pages of
+  ``page_size`` positions, laid out ``[line, page, Hkv, page_size, D]`` so that one
+  head's positions of a page are contiguous; each slot maps its logical pages to pool
+  pages.  A group with a window gives pages back as soon as no later query can see them;
+* a **state group** is ``[line, slot, *shape]`` and a slot's part is zeroed when the
+  slot is handed out;
+* pages are not cleared when a slot is freed or handed out again.
+
+All bookkeeping is on the host and works without a GPU; only the storage is on the
+device.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from ..errors import CacheFullError, RocmlError
+from ..parts.base import KVCacheRequest, StateRequest
+
+PAGE_SIZE = 64
+
+
+def pages_for(length: int, page_size: int = PAGE_SIZE) -> int:
+    return (length + page_size - 1) // page_size
+
+
+class SlotAllocator:
+    """Hands out the integers ``0 .. n-1``; lowest free number first, so that freed
+    slots are used again at once."""
+
+    def __init__(self, n_slots: int):
+        self.n_slots = n_slots
+        self._free = list(range(n_slots - 1, -1, -1))
+        self._live = set()
+
+    def alloc(self) -> int:
+        if not self._free:
+            raise CacheFullError(f"all {self.n_slots} sequence slots are in use")
+        slot = self._free.pop()
+        self._live.add(slot)
+        return slot
+
+    def free(self, slot: int) -> None:
+        if slot not in self._live:
+            raise RocmlError(f"slot {slot} is not in use (freed twice, or never handed out)")
+        self._live.remove(slot)
+        self._free.append(slot)
+        self._free.sort(reverse=True)
+
+    def is_live(self, slot: int) -> bool:
+        return slot in self._live
+
+    @property
+    def n_free(self) -> int:
+        return len(self._free)
+
+    @property
+    def live(self):
+        return frozenset(self._live)
+
+
+class KVGroup:
+    """Paged keys and values of the cache lines that share one ``KVCacheRequest``."""
+
+    def __init__(self, name: str, request: KVCacheRequest, n_lines: int, n_pages: int,
+                 page_size: int, dtype: torch.dtype, device):
+        self.name = name
+        self.request = request
+        self.n_lines = n_lines
+        self.n_pages = n_pages
+        self.page_size = page_size
+        shape = (n_lines, n_pages, request.n_kv_heads, page_size, request.head_dim)
+        self.k = torch.empty(shape, dtype=dtype, device=device)
+        self.v = torch.empty(shape, dtype=dtype, device=device)
+        self._free = list(range(n_pages - 1, -1, -1))
+        self._pages: Dict[int, List[int]] = {}   # slot -> logical page -> pool page, -1 once released
+
+    # -- bookkeeping -----------------------------------------------------------------
+    @property
+    def n_free_pages(self) -> int:
+        return len(self._free)
+
+    def open(self, slot: int) -> None:
+        self._pages[slot] = []
+
+    def pages_needed(self, slot: int, new_len: int) -> int:
+        return max(0, pages_for(new_len, self.page_size) - len(self._pages[slot]))
+
+    def grow(self, slot: int, new_len: int) -> None:
+        need = self.pages_needed(slot, new_len)
+        if need > len(self._free):
+            raise CacheFullError(f"cache group {self.name}: {need} more pages of {self.page_size} "
+                                 f"positions are needed, {len(self._free)} of {self.n_pages} are free")
+        table = self._pages[slot]
+        for _ in range(need):
+            table.append(self._free.pop())
+
+    def trim(self, slot: int, length: int) -> None:
+        """After a sequence reached ``length``: a group with a window releases the pages
+        whose positions no query at ``length`` or later can see."""
+        w = self.request.window
+        if w is None:
+            return
+        first_needed = max(0, length - w + 1) // self.page_size
+        table = self._pages[slot]
+        for i in range(min(first_needed, len(table))):
+            if table[i] >= 0:
+                self._free.append(table[i])
+                table[i] = -1
+
+    def close(self, slot: int) -> None:
+        for page in self._pages.pop(slot):
+            if page >= 0:
+                self._free.append(page)
+
+    def page_table(self, slot: int) -> List[int]:
+        return self._pages[slot]
+
+    def check(self) -> None:
+        """No page lost, none held twice, none both free and held."""
+        held = [p for table in self._pages.values() for p in table if p >= 0]
+        everything = sorted(held + self._free)
+        if everything != list(range(self.n_pages)):
+            raise RocmlError(f"cache group {self.name}: pages out of balance "
+                             f"({len(held)} held, {len(self._free)} free, {self.n_pages} in all)")
+
+    def bytes_per_token(self) -> int:
+        r = self.request
+        return 2 * self.n_lines * r.n_kv_heads * r.head_dim * self.k.element_size()
+
+
+class StateGroup:
+    """Fixed-size per-sequence state of the cache lines that share one ``StateRequest``."""
+
+    def __init__(self, name: str, request: StateRequest, n_lines: int, n_slots: int, device):
+        self.name = name
+        self.request = request
+        self.n_lines = n_lines
+        self.state = torch.zeros((n_lines, n_slots) + tuple(request.shape), dtype=request.dtype, device=device)
+
+    def open(self, slot: int) -> None:
+        self.state[:, slot].zero_()
+
+
+@dataclass
+class CacheLineView:
+    """What a mixer sees of the cache for one execution of its layer in one step."""
+    group: object
+    line: int
+    k: Optional[torch.Tensor] = None            # [pages, Hkv, page_size, D]
+    v: Optional[torch.Tensor] = None
+    block_table: Optional[torch.Tensor] = None  # [B, width] int32 on the device, per step
+    state: Optional[torch.Tensor] = None        # [slots, *shape]
+    slots: Optional[torch.Tensor] = None        # [B] int32 on the device, per step
+
+
+class Cache:
+    """Slots, groups and the mapping from schedule entries to cache lines.
+
+    ``requests[i]`` is what schedule entry ``i`` asks for (``None`` for an entry that
+    owns no cache line).  ``max_tokens`` is the number of positions live sequences may
+    hold together, each rounded up to whole pages; ``max_seqs`` bounds the live sequences."""
+
+    def __init__(self, requests: Sequence[Optional[object]], max_tokens: int, dtype: torch.dtype,
+                 device, max_seqs: Optional[int] = None, page_size: int = PAGE_SIZE):
+        self.page_size = page_size
+        self.n_pages = max(1, pages_for(max_tokens, page_size))
+        self.max_seqs = max_seqs if max_seqs is not None else self.n_pages
+        self.slots = SlotAllocator(self.max_seqs)
+        self.lengths: Dict[int, int] = {}
+        self.kv_groups: List[KVGroup] = []
+        self.state_groups: List[StateGroup] = []
+        self._line_of: Dict[int, Tuple[object, int]] = {}
+        by_request: Dict[object, List[int]] = {}
+        for entry, req in enumerate(requests):
+            if req is not None:
+                by_request.setdefault(req, []).append(entry)
+        for req, entries in by_request.items():
+            if isinstance(req, KVCacheRequest):
+                n_pages = self.n_pages
+                if req.window is not None and max_seqs is not None:
+                    n_pages = min(n_pages, max_seqs * (pages_for(req.window, page_size) + 1))
+                name = f"kv{len(self.kv_groups)}" + ("" if req.window is None else f"w{req.window}")
+                group = KVGroup(name, req, len(entries), n_pages, page_size, dtype, device)
+                self.kv_groups.append(group)
+            elif isinstance(req, StateRequest):
+                group = StateGroup(f"state{len(self.state_groups)}", req, len(entries), self.max_seqs, device)
+                self.state_groups.append(group)
+            else:
+                raise RocmlError(f"unknown cache request {req!r}")
+            for line, entry in enumerate(entries):
+                self._line_of[entry] = (group, line)
+
+    # -- sequences -------------------------------------------------------------------
+    def new_sequence(self) -> int:
+        slot = self.slots.alloc()
+        self.lengths[slot] = 0
+        for g in self.kv_groups:
+            g.open(slot)
+        for g in self.state_groups:
+            g.open(slot)
+        return slot
+
+    def free_sequence(self, slot: int) -> None:
+        self.slots.free(slot)
+        del self.lengths[slot]
+        for g in self.kv_groups:
+            g.close(slot)
+
+    def length(self, slot: int) -> int:
+        return self.lengths[slot]
+
+    def reserve(self, slots: Sequence[int], new_lens: Sequence[int]) -> None:
+        """Pages for every sequence to reach its new length, or none at all."""
+        for g in self.kv_groups:
+            need = sum(g.pages_needed(s, n) for s, n in zip(slots, new_lens))
+            if need > g.n_free_pages:
+                raise CacheFullError(
+                    f"cache group {g.name}: the step needs {need} more pages of {g.page_size} "
+                    f"positions, {g.n_free_pages} of {g.n_pages} are free")
+        for g in self.kv_groups:
+            for s, n in zip(slots, new_lens):
+                g.grow(s, n)
+
+    def commit(self, slots: Sequence[int], new_lens: Sequence[int]) -> None:
+        for s, n in zip(slots, new_lens):
+            self.lengths[s] = n
+            for g in self.kv_groups:
+                g.trim(s, n)
+
+    # -- per step --------------------------------------------------------------------
+    def block_table(self, group: KVGroup, slots: Sequence[int], width: int) -> np.ndarray:
+        table = np.full((len(slots), width), -1, dtype=np.int32)
+        for row, slot in enumerate(slots):
+            pages = group.page_table(slot)
+            table[row, :len(pages)] = pages
+        return table
+
+    def table_width(self, slots: Sequence[int]) -> int:
+        return max([1] + [len(g.page_table(s)) for g in self.kv_groups for s in slots])
+
+    def line(self, entry: int) -> Tuple[object, int]:
+        return self._line_of[entry]
+
+    def has_line(self, entry: int) -> bool:
+        return entry in self._line_of
+
+    def check(self) -> None:
+        for g in self.kv_groups:
+            g.check()
+            if set(g._pages) != set(self.lengths):
+                raise RocmlError(f"cache group {g.name}: slots and page tables disagree")
+        if set(self.lengths) != set(self.slots.live):
+            raise RocmlError("slot allocator and length table disagree")
+
+    def bytes_per_token(self) -> int:
+        """``2 * lines * Hkv * D * bytes`` summed over groups (rocml/src/budget/mod.rs:47-59)."""
+        return sum(g.bytes_per_token() for g in self.kv_groups)

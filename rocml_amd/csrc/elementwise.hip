@@ -1,0 +1,291 @@
+// Memory-bound kernels of the decoder for gfx950 (wave64): embedding gather, RMSNorm,
+// SwiGLU, rotation tables, and the fused per-head norm + rotation + cache append.
+// Norm statistics, angles and the SiLU are computed in 32-bit (angles in 64-bit) whatever
+// the storage type is.
+#include "common.h"
+
+ROCML_LAST_ERROR_FN(elementwise)
+
+constexpr int EW_BLOCK = 256;
+
+// ---- embedding -------------------------------------------------------------------
+// out[t, :] = float(table[ids[t], :]) * scale  (rocml-kernels/kernels/embedding.hip:6-18;
+// the reference has no scale, callers pass 1).
+template <typename T>
+__global__ void embed_gather_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                                    float* __restrict__ out, int hidden, int vocab, float scale) {
+    int t = blockIdx.x;
+    int id = ids[t];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    const T* row = table + (size_t)id * hidden;
+    float* o = out + (size_t)t * hidden;
+    for (int i = threadIdx.x; i < hidden; i += EW_BLOCK) o[i] = Elem<T>::load(row + i) * scale;
+}
+
+ROCML_EXPORT int rocml_embed_gather(const void* table, int table_dtype, const int* ids, float* out,
+                                    int n_tokens, int hidden, int vocab, float scale,
+                                    hipStream_t stream) {
+    ROCML_REQUIRE(n_tokens >= 0 && hidden > 0 && vocab > 0, "embed_gather: bad sizes T=%d H=%d V=%d",
+                  n_tokens, hidden, vocab);
+    if (n_tokens == 0) return 0;
+    if (table_dtype == ROCML_F32)
+        embed_gather_kernel<float><<<n_tokens, EW_BLOCK, 0, stream>>>((const float*)table, ids, out,
+                                                                      hidden, vocab, scale);
+    else if (table_dtype == ROCML_BF16)
+        embed_gather_kernel<bf16_t><<<n_tokens, EW_BLOCK, 0, stream>>>((const bf16_t*)table, ids, out,
+                                                                       hidden, vocab, scale);
+    else
+        return rocml_fail("embed_gather: unknown dtype code %d", table_dtype);
+    ROCML_CHECK_LAUNCH("embed_gather");
+    return 0;
+}
+
+// ---- block reduction -------------------------------------------------------------
+// Sum over a block of EW_BLOCK threads in a fixed order: lanes by butterfly, waves in order.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+    v = wave_sum(v);
+    int wave = threadIdx.x / WAVE;
+    __syncthreads();
+    if ((threadIdx.x & (WAVE - 1)) == 0) scratch[wave] = v;
+    __syncthreads();
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < EW_BLOCK / WAVE; ++w) total += scratch[w];
+    return total;
+}
+
+// ---- RMSNorm ---------------------------------------------------------------------
+// out[r, i] = x[src(r), i] * (1/sqrt(sum(x^2)/n + eps)) * gain[i]
+// (rocml-kernels/kernels/rmsnorm.hip:18-42).  `rows` optionally gathers source rows.
+template <typename TO>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ gain,
+                               TO* __restrict__ out, const int* __restrict__ rows, int n, float eps) {
+    __shared__ float scratch[EW_BLOCK / WAVE];
+    int r = blockIdx.x;
+    int src = rows ? rows[r] : r;
+    const float* xin = x + (size_t)src * n;
+    TO* o = out + (size_t)r * n;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += EW_BLOCK) {
+        float v = xin[i];
+        ss = fmaf(v, v, ss);
+    }
+    float total = block_sum(ss, scratch);
+    float inv = 1.0f / sqrtf(total / (float)n + eps);
+    for (int i = threadIdx.x; i < n; i += EW_BLOCK) Elem<TO>::store(o + i, xin[i] * inv * gain[i]);
+}
+
+ROCML_EXPORT int rocml_rmsnorm(const float* x, const float* gain, void* out, int out_dtype,
+                               const int* rows, int n_rows, int n, float eps, hipStream_t stream) {
+    ROCML_REQUIRE(n_rows >= 0 && n > 0, "rmsnorm: bad sizes rows=%d n=%d", n_rows, n);
+    ROCML_REQUIRE(eps > 0.f, "rmsnorm: eps must be positive, got %g", (double)eps);
+    if (n_rows == 0) return 0;
+    if (out_dtype == ROCML_F32)
+        rmsnorm_kernel<float><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (float*)out, rows, n, eps);
+    else if (out_dtype == ROCML_BF16)
+        rmsnorm_kernel<bf16_t><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (bf16_t*)out, rows, n, eps);
+    else
+        return rocml_fail("rmsnorm: unknown dtype code %d", out_dtype);
+    ROCML_CHECK_LAUNCH("rmsnorm");
+    return 0;
+}
+
+// ---- gated activation ------------------------------------------------------------
+// out[t, i] = silu(gu[t, i]) * gu[t, inter + i],  silu(g) = g / (1 + exp(-g))
+// (rocml-kernels/kernels/silu_mul.hip:12-20).  Gate and up halves lie side by side in a row.
+template <typename TI, typename TO>
+__global__ void swiglu_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inter,
+                              long long total) {
+    long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
+    if (idx >= total) return;
+    long long t = idx / inter;
+    int i = (int)(idx - t * inter);
+    const TI* row = gu + (size_t)t * 2 * inter;
+    float g = Elem<TI>::load(row + i);
+    float u = Elem<TI>::load(row + inter + i);
+    Elem<TO>::store(out + idx, g / (1.0f + expf(-g)) * u);
+}
+
+ROCML_EXPORT int rocml_swiglu(const void* gu, int in_dtype, void* out, int out_dtype, int n_tokens,
+                              int inter, hipStream_t stream) {
+    ROCML_REQUIRE(n_tokens >= 0 && inter > 0, "swiglu: bad sizes T=%d I=%d", n_tokens, inter);
+    long long total = (long long)n_tokens * inter;
+    if (total == 0) return 0;
+    int grid = ceil_div(total, EW_BLOCK);
+    if (in_dtype == ROCML_F32 && out_dtype == ROCML_F32)
+        swiglu_kernel<float, float><<<grid, EW_BLOCK, 0, stream>>>((const float*)gu, (float*)out, inter, total);
+    else if (in_dtype == ROCML_F32 && out_dtype == ROCML_BF16)
+        swiglu_kernel<float, bf16_t><<<grid, EW_BLOCK, 0, stream>>>((const float*)gu, (bf16_t*)out, inter, total);
+    else if (in_dtype == ROCML_BF16 && out_dtype == ROCML_BF16)
+        swiglu_kernel<bf16_t, bf16_t><<<grid, EW_BLOCK, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, total);
+    else
+        return rocml_fail("swiglu: unsupported dtype pair in=%d out=%d", in_dtype, out_dtype);
+    ROCML_CHECK_LAUNCH("swiglu");
+    return 0;
+}
+
+// ---- rotation tables -------------------------------------------------------------
+// cos/sin of pos * inv_freq[i] for every token of a step, angle formed in 64-bit so that the
+// 32-bit table is exact to rounding (the reference forms the angle in 32-bit,
+// rocml-kernels/kernels/rope.hip:23-27).  inv_freq[i] = theta^(-2i/rot_dim) comes from the host.
+__global__ void rope_table_kernel(const int* __restrict__ pos, const double* __restrict__ inv_freq,
+                                  float* __restrict__ cos_t, float* __restrict__ sin_t, int half,
+                                  long long total) {
+    long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
+    if (idx >= total) return;
+    long long t = idx / half;
+    int i = (int)(idx - t * half);
+    double a = (double)pos[t] * inv_freq[i];
+    cos_t[idx] = (float)cos(a);
+    sin_t[idx] = (float)sin(a);
+}
+
+ROCML_EXPORT int rocml_rope_table(const int* pos, const double* inv_freq, float* cos_t, float* sin_t,
+                                  int n_tokens, int half, hipStream_t stream) {
+    ROCML_REQUIRE(n_tokens >= 0 && half > 0, "rope_table: bad sizes T=%d half=%d", n_tokens, half);
+    long long total = (long long)n_tokens * half;
+    if (total == 0) return 0;
+    rope_table_kernel<<<ceil_div(total, EW_BLOCK), EW_BLOCK, 0, stream>>>(pos, inv_freq, cos_t, sin_t,
+                                                                           half, total);
+    ROCML_CHECK_LAUNCH("rope_table");
+    return 0;
+}
+
+// ---- per-head norm + rotation + cache append -------------------------------------
+// One wave per (token, head row) of the packed projection output [T, (Hq + 2 Hkv) * D]:
+// q and k rows are normalised over D with one gain vector each
+// (rocml/src/forward/attention.rs:105-123), rotated with NEOX pairing (i, i + rot/2)
+// (rocml-kernels/kernels/rope.hip:18-33); q goes to q_out, k and v go straight into the
+// paged cache at the token's position (rocml-kernels/kernels/chunk_reshape.hip:37-74 is the
+// reference's separate scatter).  Cache layout: [page, Hkv, page_size, D].
+constexpr int QK_MAX_PER_LANE = 8;   // D <= 512
+constexpr int QK_WAVES = EW_BLOCK / WAVE;
+
+template <typename TI, typename TO>
+__global__ void qk_norm_rope_append_kernel(
+    const TI* __restrict__ qkv, int ld, int n_tokens, int hq, int hkv, int d,
+    const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot,
+    TO* __restrict__ q_out, TO* __restrict__ kcache, TO* __restrict__ vcache,
+    const int* __restrict__ block_table, int bt_width, const int* __restrict__ token_seq,
+    const int* __restrict__ token_pos, int page_size, int write_kv) {
+    extern __shared__ float stage[];   // [QK_WAVES][d]
+    int wave = threadIdx.x / WAVE;
+    int lane = threadIdx.x & (WAVE - 1);
+    int rows_per_token = hq + 2 * hkv;
+    long long row = (long long)blockIdx.x * QK_WAVES + wave;
+    bool active = row < (long long)n_tokens * rows_per_token;
+    int t = active ? (int)(row / rows_per_token) : 0;
+    int r = active ? (int)(row - (long long)t * rows_per_token) : 0;
+    int kind = r < hq ? 0 : (r < hq + hkv ? 1 : 2);   // q, k, v
+    if (!write_kv && kind != 0) active = false;
+    const TI* src = qkv + (size_t)t * ld + (size_t)r * d;
+    float v[QK_MAX_PER_LANE];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < QK_MAX_PER_LANE; ++j) {
+        int e = lane + j * WAVE;
+        v[j] = (active && e < d) ? Elem<TI>::load(src + e) : 0.f;
+        ss = fmaf(v[j], v[j], ss);
+    }
+    const float* gain = kind == 0 ? q_gain : (kind == 1 ? k_gain : nullptr);
+    if (gain) {
+        float inv = 1.0f / sqrtf(wave_sum(ss) / (float)d + eps);
+#pragma unroll
+        for (int j = 0; j < QK_MAX_PER_LANE; ++j) {
+            int e = lane + j * WAVE;
+            if (e < d) v[j] = v[j] * inv * gain[e];
+        }
+    }
+    bool rotate = cos_t != nullptr && kind != 2;
+    float* mine = stage + (size_t)wave * d;
+    if (rotate) {
+#pragma unroll
+        for (int j = 0; j < QK_MAX_PER_LANE; ++j) {
+            int e = lane + j * WAVE;
+            if (e < d) mine[e] = v[j];
+        }
+    }
+    __syncthreads();
+    if (rotate) {
+        int half = rot / 2;
+        const float* c = cos_t + (size_t)t * half;
+        const float* s = sin_t + (size_t)t * half;
+#pragma unroll
+        for (int j = 0; j < QK_MAX_PER_LANE; ++j) {
+            int e = lane + j * WAVE;
+            if (e < rot) {
+                if (e < half) v[j] = v[j] * c[e] - mine[e + half] * s[e];
+                else v[j] = mine[e - half] * s[e - half] + v[j] * c[e - half];
+            }
+        }
+    }
+    if (!active) return;
+    TO* dst;
+    if (kind == 0) {
+        dst = q_out + ((size_t)t * hq + r) * d;
+    } else {
+        int head = kind == 1 ? r - hq : r - hq - hkv;
+        int pos = token_pos[t];
+        int page = block_table[(size_t)token_seq[t] * bt_width + pos / page_size];
+        if (page < 0) return;
+        TO* base = kind == 1 ? kcache : vcache;
+        dst = base + (((size_t)page * hkv + head) * page_size + pos % page_size) * d;
+    }
+#pragma unroll
+    for (int j = 0; j < QK_MAX_PER_LANE; ++j) {
+        int e = lane + j * WAVE;
+        if (e < d) Elem<TO>::store(dst + e, v[j]);
+    }
+}
+
+ROCML_EXPORT int rocml_qk_norm_rope_append(
+    const void* qkv, int in_dtype, int ld, int n_tokens, int hq, int hkv, int d, const float* q_gain,
+    const float* k_gain, float eps, const float* cos_t, const float* sin_t, int rot, void* q_out,
+    void* kcache, void* vcache, int out_dtype, const int* block_table, int bt_width,
+    const int* token_seq, const int* token_pos, int page_size, int write_kv, hipStream_t stream) {
+    ROCML_REQUIRE(n_tokens >= 0 && hq > 0 && hkv > 0 && d > 0, "qk_norm_rope_append: bad sizes");
+    ROCML_REQUIRE(d <= QK_MAX_PER_LANE * WAVE, "qk_norm_rope_append: head_dim %d exceeds %d", d,
+                  QK_MAX_PER_LANE * WAVE);
+    ROCML_REQUIRE(ld >= (hq + 2 * hkv) * d || (!write_kv && ld >= hq * d),
+                  "qk_norm_rope_append: row stride %d too small", ld);
+    ROCML_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "qk_norm_rope_append: rot_dim %d must be even and <= %d", rot, d);
+    ROCML_REQUIRE(!write_kv || (page_size > 0 && bt_width > 0 && block_table && kcache && vcache),
+                  "qk_norm_rope_append: cache arguments missing");
+    if (n_tokens == 0) return 0;
+    long long rows = (long long)n_tokens * (hq + 2 * hkv);
+    int grid = ceil_div(rows, QK_WAVES);
+    size_t lds = (size_t)QK_WAVES * d * sizeof(float);
+#define LAUNCH(TI, TO)                                                                          \
+    qk_norm_rope_append_kernel<TI, TO><<<grid, EW_BLOCK, lds, stream>>>(                        \
+        (const TI*)qkv, ld, n_tokens, hq, hkv, d, q_gain, k_gain, eps, cos_t, sin_t, rot,       \
+        (TO*)q_out, (TO*)kcache, (TO*)vcache, block_table, bt_width, token_seq, token_pos,      \
+        page_size, write_kv)
+    if (in_dtype == ROCML_F32 && out_dtype == ROCML_F32) LAUNCH(float, float);
+    else if (in_dtype == ROCML_F32 && out_dtype == ROCML_BF16) LAUNCH(float, bf16_t);
+    else if (in_dtype == ROCML_BF16 && out_dtype == ROCML_BF16) LAUNCH(bf16_t, bf16_t);
+    else return rocml_fail("qk_norm_rope_append: unsupported dtype pair in=%d out=%d", in_dtype, out_dtype);
+#undef LAUNCH
+    ROCML_CHECK_LAUNCH("qk_norm_rope_append");
+    return 0;
+}
+
+// ---- residual add ----------------------------------------------------------------
+// x += y  (rocml-kernels/kernels/elementwise.hip:7-12); parts without a fused epilogue use it.
+template <typename T>
+__global__ void add_into_kernel(float* __restrict__ x, const T* __restrict__ y, long long total) {
+    long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
+    if (idx < total) x[idx] += Elem<T>::load(y + idx);
+}
+
+ROCML_EXPORT int rocml_add_into(float* x, const void* y, int y_dtype, long long total,
+                                hipStream_t stream) {
+    ROCML_REQUIRE(total >= 0, "add_into: negative size");
+    if (total == 0) return 0;
+    int grid = ceil_div(total, EW_BLOCK);
+    if (y_dtype == ROCML_F32) add_into_kernel<float><<<grid, EW_BLOCK, 0, stream>>>(x, (const float*)y, total);
+    else if (y_dtype == ROCML_BF16) add_into_kernel<bf16_t><<<grid, EW_BLOCK, 0, stream>>>(x, (const bf16_t*)y, total);
+    else return rocml_fail("add_into: unknown dtype code %d", y_dtype);
+    ROCML_CHECK_LAUNCH("add_into");
+    return 0;
+}

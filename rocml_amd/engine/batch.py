@@ -1,0 +1,66 @@
+"""What one step of the engine works on: the tokens of a batch, packed.
+
+The reference's two entry points take one sequence and an implicit position
+(rocml/src/forward/chunk_forward.rs:62, rocml/src/forward/mod.rs:236).  A step here
+takes several sequences with unequal numbers of new tokens; they are packed one after
+another, and every token carries its sequence and its absolute position, so rotation,
+cache append and the causal bound need nothing else.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from .workspace import Workspace
+
+
+@dataclass
+class StepEntry:
+    """New tokens of one sequence and the places among them whose logits are wanted."""
+    slot: int
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+@dataclass
+class StepContext:
+    n_tokens: int
+    n_seqs: int
+    token_ids: torch.Tensor      # [T] int32
+    token_seq: torch.Tensor      # [T] int32: index of the token's sequence in this step
+    token_pos: torch.Tensor      # [T] int32: absolute position
+    cu_seqlens: torch.Tensor     # [B + 1] int32: where each sequence's tokens start
+    seq_lens: torch.Tensor       # [B] int32: sequence length after this step
+    seq_slots: torch.Tensor      # [B] int32: cache slot of each sequence
+    max_new: int                 # most new tokens of any sequence
+    max_len: int                 # longest sequence after this step
+    workspace: Workspace
+    memo: Dict = field(default_factory=dict)
+
+    @property
+    def is_decode(self) -> bool:
+        return self.max_new == 1
+
+
+def pack_step(slots: Sequence[int], starts: Sequence[int], tokens: Sequence[Sequence[int]]):
+    """Host arrays of a packed step: ids, sequence index and position per token, offsets,
+    final lengths."""
+    counts = [len(t) for t in tokens]
+    total = sum(counts)
+    ids = np.empty(total, dtype=np.int32)
+    seq = np.empty(total, dtype=np.int32)
+    pos = np.empty(total, dtype=np.int32)
+    cu = np.zeros(len(tokens) + 1, dtype=np.int32)
+    at = 0
+    for b, (start, toks) in enumerate(zip(starts, tokens)):
+        n = len(toks)
+        ids[at:at + n] = toks
+        seq[at:at + n] = b
+        pos[at:at + n] = np.arange(start, start + n, dtype=np.int32)
+        at += n
+        cu[b + 1] = at
+    lens = np.asarray([s + c for s, c in zip(starts, counts)], dtype=np.int32)
+    return ids, seq, pos, cu, lens, np.asarray(slots, dtype=np.int32)

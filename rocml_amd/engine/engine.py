@@ -1,0 +1,151 @@
+"""The step function: a batch of sequences, their new tokens, logits at wanted places.
+
+One entry point replaces the reference's pair ``forward_chunk`` / ``forward_token``
+(rocml/src/forward/chunk_forward.rs:62-189, rocml/src/forward/mod.rs:246-387): a step
+runs exactly the tokens it is given, as one packed batch, on top of what earlier steps
+left in the cache, and returns 32-bit logits only for the rows that were asked for
+(the reference computes the last row only, chunk_forward.rs:143-184).  A sequence that
+would pass the model's positions is an error, never a truncation
+(rocml/src/forward/mod.rs:253-258).  Long steps are cut into pieces of at most
+``max_step_tokens`` tokens internally, as the reference cuts prompts at 512
+(chunk_forward.rs:41-52); the cut is invisible because every piece reads the cache.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache import Cache
+from ..errors import ContextOverflowError, RocmlError
+from .batch import StepContext, StepEntry, pack_step
+from .model import DecoderModel
+from .workspace import Workspace
+
+
+def _bucket(n: int) -> int:
+    b = 1
+    while b < n:
+        b *= 2
+    return b
+
+
+class Engine:
+    def __init__(self, model: DecoderModel, max_tokens: int, max_seqs: Optional[int] = None,
+                 max_step_tokens: int = 8192):
+        if model.embed is None:
+            raise RocmlError("the model has no weights bound")
+        self.model = model
+        self.cache: Cache = model.new_cache(max_tokens, max_seqs)
+        self.workspace = Workspace(model.device)
+        self.max_step_tokens = max_step_tokens
+        self.steps_run = 0
+
+    # -- sequences -----------------------------------------------------------------------
+    def new_sequence(self) -> int:
+        return self.cache.new_sequence()
+
+    def release(self, slot: int) -> None:
+        self.cache.free_sequence(slot)
+
+    def length(self, slot: int) -> int:
+        return self.cache.length(slot)
+
+    # -- the step ------------------------------------------------------------------------
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Runs the entries' tokens; returns ``[n_wanted, vocab]`` 32-bit logits on the
+        device in the order of the entries and of their ``want`` lists, or None when
+        nothing is wanted.  The result is a buffer of the engine and holds until the next
+        step."""
+        spec = self.model.spec
+        if not entries:
+            return None
+        slots = [e.slot for e in entries]
+        if len(set(slots)) != len(slots):
+            raise RocmlError("a sequence appears twice in one step")
+        starts, new_lens = [], []
+        for e in entries:
+            if not self.cache.slots.is_live(e.slot):
+                raise RocmlError(f"slot {e.slot} is not a live sequence")
+            if len(e.tokens) == 0:
+                raise RocmlError("a step entry needs at least one token")
+            for t in e.tokens:
+                if not 0 <= int(t) < spec.vocab:
+                    raise RocmlError(f"token id {t} is outside the vocabulary of {spec.vocab}")
+            for w in e.want:
+                if not 0 <= int(w) < len(e.tokens):
+                    raise RocmlError(f"wanted place {w} is outside the entry's {len(e.tokens)} tokens")
+            start = self.cache.length(e.slot)
+            if start + len(e.tokens) > spec.max_positions:
+                raise ContextOverflowError(
+                    f"sequence would reach {start + len(e.tokens)} positions; the model has "
+                    f"{spec.max_positions}")
+            starts.append(start)
+            new_lens.append(start + len(e.tokens))
+        self.cache.reserve(slots, new_lens)
+
+        total = sum(len(e.tokens) for e in entries)
+        n_want_total = sum(len(e.want) for e in entries)
+        if total <= self.max_step_tokens:
+            logits = self._run_piece(slots, starts, [list(e.tokens) for e in entries],
+                                     [list(e.want) for e in entries])
+            self.cache.commit(slots, new_lens)
+            self.steps_run += 1
+            return logits
+
+        # Cut the packed tokens into pieces; a sequence may straddle pieces.
+        result = None
+        if n_want_total:
+            result = torch.empty((n_want_total, spec.vocab), dtype=torch.float32, device=self.model.device)
+        want_base = np.cumsum([0] + [len(e.want) for e in entries])
+        done = [0] * len(entries)
+        while any(done[i] < len(e.tokens) for i, e in enumerate(entries)):
+            room = self.max_step_tokens
+            p_slots, p_starts, p_tokens, p_want, p_dest = [], [], [], [], []
+            for i, e in enumerate(entries):
+                left = len(e.tokens) - done[i]
+                if left == 0 or room == 0:
+                    continue
+                take = min(left, room)
+                lo, hi = done[i], done[i] + take
+                wanted = [(k, w - lo) for k, w in enumerate(e.want) if lo <= w < hi]
+                p_slots.append(e.slot)
+                p_starts.append(starts[i] + lo)
+                p_tokens.append(list(e.tokens[lo:hi]))
+                p_want.append([w for _, w in wanted])
+                p_dest.extend(int(want_base[i]) + k for k, _ in wanted)
+                done[i] = hi
+                room -= take
+            logits = self._run_piece(p_slots, p_starts, p_tokens, p_want)
+            if logits is not None:
+                result[torch.as_tensor(p_dest, device=self.model.device)] = logits
+            self.cache.commit(p_slots, [s + len(t) for s, t in zip(p_starts, p_tokens)])
+        self.steps_run += 1
+        return result
+
+    def _run_piece(self, slots: List[int], starts: List[int], tokens: List[List[int]],
+                   want: List[List[int]]) -> Optional[torch.Tensor]:
+        ids, seq, pos, cu, lens, slot_arr = pack_step(slots, starts, tokens)
+        want_rows = np.asarray([int(cu[b]) + w for b, ws_ in enumerate(want) for w in ws_], dtype=np.int32)
+        width = _bucket(self.cache.table_width(slots))
+        tables = [self.cache.block_table(g, slots, width) for g in self.cache.kv_groups]
+        # One upload for all integer tables of the step.
+        parts = [ids, seq, pos, cu, lens, slot_arr, want_rows] + [t.reshape(-1) for t in tables]
+        host = np.concatenate(parts) if parts else np.zeros(0, np.int32)
+        meta = self.workspace.get("step.meta", (max(host.size, 1),), torch.int32)
+        meta[:host.size].copy_(torch.from_numpy(host))
+        views, at = [], 0
+        for p in parts:
+            views.append(meta[at:at + p.size])
+            at += p.size
+        d_ids, d_seq, d_pos, d_cu, d_lens, d_slots, d_want = views[:7]
+        block_tables: Dict[str, torch.Tensor] = {}
+        for g, v in zip(self.cache.kv_groups, views[7:]):
+            block_tables[g.name] = v.view(len(slots), width)
+        step = StepContext(n_tokens=int(ids.size), n_seqs=len(slots), token_ids=d_ids, token_seq=d_seq,
+                           token_pos=d_pos, cu_seqlens=d_cu, seq_lens=d_lens, seq_slots=d_slots,
+                           max_new=max(len(t) for t in tokens), max_len=int(lens.max()),
+                           workspace=self.workspace)
+        return self.model.forward(step, self.cache, block_tables, d_want if want_rows.size else None,
+                                  int(want_rows.size))

@@ -1,0 +1,113 @@
+"""A decoder built from a ``ModelSpec``: embedding, the layers in schedule order, final
+norm and output matrix.  It holds no sizes of its own and no knowledge of any
+architecture; the data flow is the reference's (rocml/src/forward/chunk_forward.rs:96-184):
+embedding, blocks, then norm and output product only for the rows whose logits are wanted.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from .. import ops
+from ..cache import Cache, CacheLineView, KVGroup
+from ..config.spec import ModelSpec
+from ..errors import ConfigError
+from ..parts import BuildContext, ParamSpec, build_block, build_norm
+from .batch import StepContext
+
+_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32,
+           torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
+
+
+def compute_dtype(name) -> torch.dtype:
+    if name not in _DTYPES:
+        raise ConfigError(f"compute type must be bfloat16 or float32, got {name!r}")
+    return _DTYPES[name]
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec, dtype, device="cuda"):
+        spec.validate()
+        self.spec = spec
+        self.dtype = compute_dtype(dtype)
+        self.device = torch.device(device)
+        ctx = BuildContext(dtype=self.dtype, device=self.device)
+        self.blocks = [build_block(b, ctx) for b in spec.layers]
+        self.final_norm = build_norm(spec.final_norm, ctx)
+        self.embed: Optional[torch.Tensor] = None
+        self.lm_head: Optional[torch.Tensor] = None
+
+    # -- parameters --------------------------------------------------------------------
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        s = self.spec
+        specs = {"embed.weight": ParamSpec((s.vocab, s.hidden))}
+        for i, block in enumerate(self.blocks):
+            for name, p in block.param_specs().items():
+                specs[f"layers.{i}.{name}"] = p
+        for name, p in self.final_norm.param_specs().items():
+            specs[f"final_norm.{name}"] = p
+        if not s.tie_lm_head:
+            specs["lm_head.weight"] = ParamSpec((s.vocab, s.hidden))
+        return specs
+
+    def storage_dtype(self, p: ParamSpec) -> torch.dtype:
+        return {"matrix": self.dtype, "gain": torch.float32, "int_table": torch.int32}[p.role]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.embed = tensors["embed.weight"]
+        # A tied output matrix is the embedding table itself, one buffer
+        # (rocml/src/weights/mod.rs:48-62 loads it twice).
+        self.lm_head = self.embed if self.spec.tie_lm_head else tensors["lm_head.weight"]
+        for i, block in enumerate(self.blocks):
+            prefix = f"layers.{i}."
+            block.bind({k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)})
+        self.final_norm.bind({k[len("final_norm."):]: v for k, v in tensors.items()
+                              if k.startswith("final_norm.")})
+
+    def weight_bytes(self) -> int:
+        total = 0
+        for name, p in self.param_specs().items():
+            n = 1
+            for d in p.shape:
+                n *= d
+            total += n * torch.empty((), dtype=self.storage_dtype(p)).element_size()
+        return total
+
+    # -- cache -------------------------------------------------------------------------
+    def cache_requests(self) -> List[Optional[object]]:
+        """What each schedule entry needs of the cache (None if it reads another's)."""
+        return [None if e.reads_cache_of is not None else self.blocks[e.layer].cache_request()
+                for e in self.spec.schedule]
+
+    def new_cache(self, max_tokens: int, max_seqs: Optional[int] = None) -> Cache:
+        return Cache(self.cache_requests(), max_tokens, self.dtype, self.device, max_seqs=max_seqs)
+
+    # -- forward -----------------------------------------------------------------------
+    def forward(self, step: StepContext, cache: Cache, block_tables: Dict[str, torch.Tensor],
+                want_rows: Optional[torch.Tensor], n_want: int) -> Optional[torch.Tensor]:
+        """Runs the step's tokens through every schedule entry; returns 32-bit logits
+        ``[n_want, vocab]`` for the token rows in ``want_rows`` (None if none are wanted)."""
+        s = self.spec
+        ws = step.workspace
+        x = ws.get("model.x", (step.n_tokens, s.hidden), torch.float32)
+        ops.embed_gather(self.embed, step.token_ids, x, s.embed_scale)
+        for i, entry in enumerate(s.schedule):
+            owner = i if entry.reads_cache_of is None else entry.reads_cache_of
+            view = None
+            if cache.has_line(owner):
+                group, line = cache.line(owner)
+                if isinstance(group, KVGroup):
+                    view = CacheLineView(group=group, line=line, k=group.k[line], v=group.v[line],
+                                         block_table=block_tables[group.name])
+                else:
+                    view = CacheLineView(group=group, line=line, state=group.state[line],
+                                         slots=step.seq_slots)
+            self.blocks[entry.layer].forward(step, x, view, owner == i)
+        if n_want == 0:
+            return None
+        xn = ws.get("model.final_xn", (n_want, s.hidden), self.dtype)
+        self.final_norm.forward(x, xn, rows=want_rows)
+        logits = ws.get("model.logits", (n_want, s.vocab), torch.float32)
+        ops.gemm(xn, self.lm_head, logits, workspace=ws.scratch())
+        return logits

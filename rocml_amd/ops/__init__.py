@@ -1,0 +1,294 @@
+"""Typed launch helpers over the compiled HIP libraries.
+
+The counterpart of the reference's ``Kernels`` struct, which loads each code object
+once and offers one typed method per kernel that fixes grid, block and LDS
+(rocml/src/forward/kernels.rs:97-229,232-720).  Here the grid is chosen inside the
+library; these helpers check devices, types and shapes, pass raw pointers and the
+current stream, and turn a nonzero status into ``KernelError`` with the library's
+message.  There is no fallback: a missing library is compiled, and if that fails the
+call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Dict, Optional
+
+import torch
+
+from ..csrc import build as _build
+from ..errors import KernelError
+
+_P = ctypes.c_void_p
+_I = ctypes.c_int
+_F = ctypes.c_float
+_LL = ctypes.c_longlong
+
+_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+
+_SIGNATURES = {
+    "elementwise": {
+        "rocml_embed_gather": [_P, _I, _P, _P, _I, _I, _I, _F, _P],
+        "rocml_rmsnorm": [_P, _P, _P, _I, _P, _I, _I, _F, _P],
+        "rocml_swiglu": [_P, _I, _P, _I, _I, _I, _P],
+        "rocml_rope_table": [_P, _P, _P, _P, _I, _I, _P],
+        "rocml_qk_norm_rope_append": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P, _P, _I, _P, _P, _P,
+                                      _I, _P, _I, _P, _P, _I, _I, _P],
+        "rocml_add_into": [_P, _P, _I, _LL, _P],
+    },
+    "gemm": {
+        "rocml_gemm": [_P, _I, _I, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _LL, _P],
+    },
+    "attention": {
+        "rocml_attention": [_P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P,
+                            _LL, _P],
+    },
+    "sampling": {
+        "rocml_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P],
+        "rocml_argmax": [_P, _I, _I, _P, _P],
+    },
+}
+
+_libs: Dict[str, ctypes.CDLL] = {}
+
+
+def library(family: str) -> ctypes.CDLL:
+    """The family's shared library, compiled on first use if it is not there."""
+    lib = _libs.get(family)
+    if lib is None:
+        lib = ctypes.CDLL(_build.ensure(family))
+        for name, argtypes in _SIGNATURES[family].items():
+            fn = getattr(lib, name)
+            fn.argtypes = argtypes
+            fn.restype = _I
+        err = getattr(lib, f"{family}_last_error")
+        err.restype = ctypes.c_char_p
+        err.argtypes = []
+        _libs[family] = lib
+    return lib
+
+
+def load_all() -> None:
+    for family in _SIGNATURES:
+        library(family)
+
+
+def _check(family: str, status: int) -> None:
+    if status != 0:
+        msg = getattr(library(family), f"{family}_last_error")().decode("utf-8", "replace")
+        raise KernelError(msg)
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _dev(*tensors: Optional[torch.Tensor]) -> None:
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise KernelError("kernel arguments must be GPU tensors; this library has no CPU path")
+        if not t.is_contiguous():
+            raise KernelError(f"kernel arguments must be contiguous, got strides {t.stride()} for shape {tuple(t.shape)}")
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise KernelError(f"unsupported element type {t.dtype}") from None
+
+
+def _want(t: torch.Tensor, dtype: torch.dtype, what: str) -> None:
+    if t.dtype != dtype:
+        raise KernelError(f"{what} must be {dtype}, got {t.dtype}")
+
+
+# ---- elementwise ---------------------------------------------------------------------
+def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
+    _dev(table, ids, out)
+    _want(ids, torch.int32, "token ids")
+    _want(out, torch.float32, "embedding output")
+    vocab, hidden = table.shape
+    n = ids.numel()
+    if out.shape != (n, hidden):
+        raise KernelError(f"embedding output is {tuple(out.shape)}, expected {(n, hidden)}")
+    _check("elementwise", library("elementwise").rocml_embed_gather(
+        _ptr(table), _code(table), _ptr(ids), _ptr(out), n, hidden, vocab, scale, _stream()))
+
+
+def rmsnorm(x: torch.Tensor, gain: torch.Tensor, eps: float, out: torch.Tensor,
+            rows: Optional[torch.Tensor] = None) -> None:
+    _dev(x, gain, out, rows)
+    _want(x, torch.float32, "norm input")
+    _want(gain, torch.float32, "norm gain")
+    n = x.shape[-1]
+    if gain.numel() != n or out.shape[-1] != n:
+        raise KernelError(f"norm sizes differ: input {n}, gain {gain.numel()}, output {out.shape[-1]}")
+    n_rows = out.numel() // n
+    if rows is not None:
+        _want(rows, torch.int32, "row indices")
+        if rows.numel() != n_rows:
+            raise KernelError("one row index per output row is needed")
+    elif x.numel() != out.numel():
+        raise KernelError("norm input and output differ in size")
+    _check("elementwise", library("elementwise").rocml_rmsnorm(
+        _ptr(x), _ptr(gain), _ptr(out), _code(out), _ptr(rows), n_rows, n, eps, _stream()))
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    _dev(gate_up, out)
+    n_tokens, inter = out.shape
+    if gate_up.shape != (n_tokens, 2 * inter):
+        raise KernelError(f"gate/up is {tuple(gate_up.shape)}, expected {(n_tokens, 2 * inter)}")
+    _check("elementwise", library("elementwise").rocml_swiglu(
+        _ptr(gate_up), _code(gate_up), _ptr(out), _code(out), n_tokens, inter, _stream()))
+
+
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> None:
+    _dev(positions, inv_freq, cos, sin)
+    _want(positions, torch.int32, "positions")
+    _want(inv_freq, torch.float64, "inverse frequencies")
+    _want(cos, torch.float32, "cos table")
+    _want(sin, torch.float32, "sin table")
+    n, half = positions.numel(), inv_freq.numel()
+    if cos.shape != (n, half) or sin.shape != (n, half):
+        raise KernelError(f"rotation tables must be {(n, half)}")
+    _check("elementwise", library("elementwise").rocml_rope_table(
+        _ptr(positions), _ptr(inv_freq), _ptr(cos), _ptr(sin), n, half, _stream()))
+
+
+def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,
+                        q_gain: Optional[torch.Tensor], k_gain: Optional[torch.Tensor], eps: float,
+                        cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rot_dim: int,
+                        q_out: torch.Tensor, k_cache: Optional[torch.Tensor],
+                        v_cache: Optional[torch.Tensor], block_table: Optional[torch.Tensor],
+                        token_seq: torch.Tensor, token_pos: torch.Tensor, write_kv: bool = True) -> None:
+    """``qkv`` is ``[T, ld]`` with q, k, v side by side (k and v may be absent when
+    ``write_kv`` is false).  Caches are ``[pages, Hkv, page_size, D]``."""
+    _dev(qkv, q_gain, k_gain, cos, sin, q_out, k_cache, v_cache, block_table, token_seq, token_pos)
+    n_tokens, ld = qkv.shape
+    for g in (q_gain, k_gain):
+        if g is not None:
+            _want(g, torch.float32, "head norm gain")
+            if g.numel() != head_dim:
+                raise KernelError(f"head norm gain has {g.numel()} values for head size {head_dim}")
+    if cos is not None:
+        if cos.shape != (n_tokens, rot_dim // 2) or sin is None or sin.shape != cos.shape:
+            raise KernelError(f"rotation tables must be {(n_tokens, rot_dim // 2)}")
+    if q_out.shape != (n_tokens, n_heads * head_dim) or token_seq.numel() != n_tokens \
+            or token_pos.numel() != n_tokens:
+        raise KernelError("q output or token tables do not match the number of tokens")
+    page_size = bt_width = 0
+    if write_kv:
+        if k_cache is None or v_cache is None or block_table is None:
+            raise KernelError("appending to the cache needs the cache and the block table")
+        if k_cache.shape[1:] != (n_kv_heads, k_cache.shape[2], head_dim) or v_cache.shape != k_cache.shape:
+            raise KernelError(f"cache shape {tuple(k_cache.shape)} does not fit {n_kv_heads} heads of {head_dim}")
+        if k_cache.dtype != q_out.dtype:
+            raise KernelError("cache and q output must share their type")
+        _want(block_table, torch.int32, "block table")
+        page_size, bt_width = k_cache.shape[2], block_table.shape[1]
+    _check("elementwise", library("elementwise").rocml_qk_norm_rope_append(
+        _ptr(qkv), _code(qkv), ld, n_tokens, n_heads, n_kv_heads, head_dim, _ptr(q_gain), _ptr(k_gain),
+        eps, _ptr(cos), _ptr(sin), rot_dim if cos is not None else 0, _ptr(q_out), _ptr(k_cache),
+        _ptr(v_cache), _code(q_out), _ptr(block_table), bt_width, _ptr(token_seq), _ptr(token_pos),
+        page_size, 1 if write_kv else 0, _stream()))
+
+
+def add_into(x: torch.Tensor, y: torch.Tensor) -> None:
+    _dev(x, y)
+    _want(x, torch.float32, "residual")
+    if x.numel() != y.numel():
+        raise KernelError("residual add of different sizes")
+    _check("elementwise", library("elementwise").rocml_add_into(_ptr(x), _ptr(y), _code(y), x.numel(), _stream()))
+
+
+# ---- matrix product ------------------------------------------------------------------
+GEMM_AUTO, GEMM_PLAIN = 0, 1
+
+
+def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
+         algo: int = GEMM_AUTO, workspace: Optional[torch.Tensor] = None) -> None:
+    """``out (+)= x @ w.T`` for ``x [M, K]``, ``w [N, K]``, ``out [M, N]`` (rows may be
+    strided views with unit inner stride)."""
+    for t in (x, w, out):
+        if not t.is_cuda:
+            raise KernelError("kernel arguments must be GPU tensors; this library has no CPU path")
+        if t.dim() != 2 or t.stride(1) != 1:
+            raise KernelError("matrix product operands must be 2-D with unit inner stride")
+    m, k = x.shape
+    n = w.shape[0]
+    if w.shape[1] != k or out.shape != (m, n):
+        raise KernelError(f"matrix product shapes do not fit: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
+    ws_ptr, ws_bytes = (None, 0) if workspace is None else (workspace.data_ptr(), workspace.numel() * workspace.element_size())
+    _check("gemm", library("gemm").rocml_gemm(
+        _ptr(x), _code(x), x.stride(0) if m > 1 else max(x.stride(0), k), _ptr(w), _code(w), w.stride(0),
+        _ptr(out), _code(out), out.stride(0) if m > 1 else max(out.stride(0), n), m, n, k,
+        1 if accumulate else 0, algo, ws_ptr, ws_bytes, _stream()))
+
+
+# ---- attention -----------------------------------------------------------------------
+ATTN_AUTO, ATTN_PLAIN = 0, 1
+
+
+def attention(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+              block_table: torch.Tensor, token_seq: torch.Tensor, token_pos: torch.Tensor,
+              n_heads: int, n_kv_heads: int, head_dim: int, scale: float, window: Optional[int] = None,
+              algo: int = ATTN_AUTO, workspace: Optional[torch.Tensor] = None) -> None:
+    _dev(q, out, k_cache, v_cache, block_table, token_seq, token_pos)
+    n_tokens = q.shape[0]
+    if q.shape != (n_tokens, n_heads * head_dim) or out.shape != q.shape or out.dtype != q.dtype:
+        raise KernelError("attention input and output must both be [tokens, heads * head_dim] of one type")
+    if k_cache.dtype != q.dtype or v_cache.shape != k_cache.shape \
+            or k_cache.shape[1] != n_kv_heads or k_cache.shape[3] != head_dim:
+        raise KernelError(f"cache {tuple(k_cache.shape)} {k_cache.dtype} does not fit the queries")
+    _want(block_table, torch.int32, "block table")
+    _want(token_seq, torch.int32, "token sequence table")
+    _want(token_pos, torch.int32, "token position table")
+    if token_seq.numel() != n_tokens or token_pos.numel() != n_tokens:
+        raise KernelError("one sequence index and one position per token are needed")
+    ws_ptr, ws_bytes = (None, 0) if workspace is None else (workspace.data_ptr(), workspace.numel() * workspace.element_size())
+    _check("attention", library("attention").rocml_attention(
+        _ptr(q), _ptr(out), _ptr(k_cache), _ptr(v_cache), _code(q), _ptr(block_table),
+        block_table.shape[1], _ptr(token_seq), _ptr(token_pos), n_tokens, n_heads, n_kv_heads, head_dim,
+        k_cache.shape[2], scale, 0 if window is None else int(window), algo, ws_ptr, ws_bytes, _stream()))
+
+
+# ---- sampling ------------------------------------------------------------------------
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
+    _dev(logits, out)
+    _want(logits, torch.float32, "logits")
+    _want(out, torch.int32, "token output")
+    batch, vocab = logits.shape
+    _check("sampling", library("sampling").rocml_argmax(_ptr(logits), batch, vocab, _ptr(out), _stream()))
+
+
+def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor,
+           out: torch.Tensor, top_k: Optional[torch.Tensor] = None, top_p: Optional[torch.Tensor] = None,
+           penalty: Optional[torch.Tensor] = None, history: Optional[torch.Tensor] = None,
+           history_len: Optional[torch.Tensor] = None) -> None:
+    _dev(logits, work, temperature, uniform, out, top_k, top_p, penalty, history, history_len)
+    _want(logits, torch.float32, "logits")
+    _want(work, torch.float32, "sampling workspace")
+    batch, vocab = logits.shape
+    if work.numel() < logits.numel():
+        raise KernelError("sampling workspace is smaller than the logits")
+    for t, dt, name in ((temperature, torch.float32, "temperature"), (uniform, torch.float32, "uniform"),
+                        (top_p, torch.float32, "top_p"), (penalty, torch.float32, "penalty"),
+                        (top_k, torch.int32, "top_k"), (history, torch.int32, "history"),
+                        (history_len, torch.int32, "history lengths"), (out, torch.int32, "token output")):
+        if t is not None:
+            _want(t, dt, name)
+            if name != "history" and t.numel() != batch:
+                raise KernelError(f"{name} needs one value per sequence")
+    if penalty is not None and (history is None or history_len is None or history.shape[0] != batch):
+        raise KernelError("a repeat penalty needs the history and its lengths")
+    _check("sampling", library("sampling").rocml_sample(
+        _ptr(logits), _ptr(work), batch, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform),
+        _ptr(penalty), _ptr(history), 0 if history is None else history.shape[1], _ptr(history_len),
+        _ptr(out), _stream()))

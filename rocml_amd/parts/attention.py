@@ -1,0 +1,89 @@
+"""Softmax attention with grouped key/value heads over the paged cache.
+
+Order of work as in the reference's layer (rocml/src/forward/attention_chunk.rs:97-330):
+projections without bias, per-head norm of q and k, rotation, append to the cache, causal
+attention with the scale applied after the dot product, output projection, residual sum.
+Here q, k and v come from one product over the concatenated weight, norm + rotation +
+append are one kernel, and the residual sum is the output product's epilogue.  Head
+counts, head size, scale, window, the optional norm and the optional position encoding
+are the spec's, nothing is fixed here.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from .. import ops
+from ..config.spec import AttentionSpec
+from ..errors import ConfigError
+from .base import BuildContext, KVCacheRequest, Mixer, ParamSpec
+from .registry import build_position, register_mixer
+
+
+class Attention(Mixer):
+    def __init__(self, spec: AttentionSpec, ctx: BuildContext):
+        if spec.n_heads % spec.n_kv_heads != 0:
+            raise ConfigError(f"{spec.n_heads} query heads are not a multiple of {spec.n_kv_heads} key/value heads")
+        if spec.qk_norm is not None and spec.qk_norm.size != spec.head_dim:
+            raise ConfigError("the per-head norm must span the head size")
+        if spec.window is not None and spec.window <= 0:
+            raise ConfigError(f"window must be positive, got {spec.window}")
+        self.spec = spec
+        self.dtype = ctx.dtype
+        self.q_dim = spec.n_heads * spec.head_dim
+        self.kv_dim = spec.n_kv_heads * spec.head_dim
+        self.position = build_position(spec.position, ctx) if spec.position is not None else None
+        self.w_qkv: Optional[torch.Tensor] = None
+        self.w_o: Optional[torch.Tensor] = None
+        self.q_gain: Optional[torch.Tensor] = None
+        self.k_gain: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        s = self.spec
+        specs = {"q_proj.weight": ParamSpec((self.q_dim, s.hidden)),
+                 "k_proj.weight": ParamSpec((self.kv_dim, s.hidden)),
+                 "v_proj.weight": ParamSpec((self.kv_dim, s.hidden)),
+                 "o_proj.weight": ParamSpec((s.hidden, self.q_dim))}
+        if s.qk_norm is not None:
+            specs["q_norm.weight"] = ParamSpec((s.head_dim,), role="gain", init="gain")
+            specs["k_norm.weight"] = ParamSpec((s.head_dim,), role="gain", init="gain")
+        return specs
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        # One [Q + 2 KV, hidden] matrix: q rows first, so a layer that only reads another
+        # layer's cache multiplies by the leading Q rows.
+        self.w_qkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"],
+                                tensors["v_proj.weight"]], dim=0).contiguous()
+        self.w_o = tensors["o_proj.weight"]
+        if self.spec.qk_norm is not None:
+            self.q_gain = tensors["q_norm.weight"]
+            self.k_gain = tensors["k_norm.weight"]
+
+    def cache_request(self) -> KVCacheRequest:
+        return KVCacheRequest(self.spec.n_kv_heads, self.spec.head_dim, self.spec.window)
+
+    def forward(self, step, xn, x_accum, cache, owns_cache: bool) -> None:
+        s = self.spec
+        n = step.n_tokens
+        ws = step.workspace
+        rows = self.q_dim + 2 * self.kv_dim if owns_cache else self.q_dim
+        qkv = ws.get("attn.qkv", (n, rows), torch.float32)
+        ops.gemm(xn, self.w_qkv[:rows], qkv, workspace=ws.scratch())
+        cos = sin = None
+        rot = 0
+        if self.position is not None:
+            cos, sin = self.position.tables(step)
+            rot = self.position.rot_dim
+        q = ws.get("attn.q", (n, self.q_dim), self.dtype)
+        eps = s.qk_norm.eps if s.qk_norm is not None else 1.0
+        ops.qk_norm_rope_append(qkv, s.n_heads, s.n_kv_heads, s.head_dim, self.q_gain, self.k_gain, eps,
+                                cos, sin, rot, q, cache.k, cache.v, cache.block_table, step.token_seq,
+                                step.token_pos, write_kv=owns_cache)
+        o = ws.get("attn.o", (n, self.q_dim), self.dtype)
+        ops.attention(q, o, cache.k, cache.v, cache.block_table, step.token_seq, step.token_pos,
+                      s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, workspace=ws.scratch())
+        ops.gemm(o, self.w_o, x_accum, accumulate=True, workspace=ws.scratch())
+
+
+register_mixer("attention", Attention)

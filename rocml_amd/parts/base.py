@@ -1,0 +1,95 @@
+"""Interfaces of the parts a decoder is put together from.
+
+The reference writes each layer as one function over one struct of weights
+(rocml/src/forward/attention.rs:30-249, rocml/src/forward/ffn.rs:17-111).  Here a
+layer is assembled from parts that know nothing about the model around them:
+
+* every part declares its parameters (``param_specs``) and receives them as device
+  tensors (``bind``);
+* a **mixer** moves information between the tokens of a sequence and may ask for
+  storage in the cache (``cache_request``): keys and values, or a state of fixed size;
+* a **feed-forward** works on each token alone;
+* a **norm** maps the 32-bit residual stream to the activation type;
+* a **position encoding** prepares per-step tables that mixers share.
+
+Mixers and feed-forwards add their result into the 32-bit residual stream they are
+handed (``x_accum``), which lets a product's epilogue do the residual sum.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Dict, Optional, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    """Shape and role of one parameter.
+
+    ``matrix``: an operand of a matrix product, held in the model's compute type.
+    ``gain``: a small vector used in 32-bit arithmetic, always held in 32-bit.
+    ``int_table``: integers, held as int32.
+    ``init`` names how random weights are drawn: ``normal`` is N(0, 0.02), ``gain`` is 1
+    (or 1 + N(0, 0.02) when jitter is asked for), ``zeros`` is 0."""
+    shape: Tuple[int, ...]
+    role: str = "matrix"
+    init: str = "normal"
+
+
+@dataclass(frozen=True)
+class BuildContext:
+    dtype: torch.dtype          # compute type: torch.bfloat16 or torch.float32
+    device: torch.device
+
+
+@dataclass(frozen=True)
+class KVCacheRequest:
+    """Keys and values per position: ``window`` is None when all positions are kept."""
+    n_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateRequest:
+    """A per-sequence state of fixed shape, zero when a sequence starts."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+class Part:
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {}
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        """Receives the tensors named by ``param_specs``, already on the device and in
+        the type their role asks for."""
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def tables(self, step: Any) -> Any:
+        """Per-step tables for the step's token positions; computed once a step."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_request(self) -> Optional[Any]:
+        return None
+
+    def forward(self, step: Any, xn: torch.Tensor, x_accum: torch.Tensor, cache: Any,
+                owns_cache: bool) -> None:
+        """Adds the mixer's output for the step's tokens into ``x_accum`` (32-bit,
+        ``[tokens, hidden]``).  ``cache`` is the view of the cache line this execution
+        uses; with ``owns_cache`` false it belongs to another execution and is read only."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, step: Any, xn: torch.Tensor, x_accum: torch.Tensor) -> None:
+        raise NotImplementedError

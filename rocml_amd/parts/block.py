@@ -1,0 +1,49 @@
+"""Arrangement of a mixer and a feed-forward into one layer.
+
+``pre_norm`` is the reference's wiring (rocml/src/forward/chunk_forward.rs:107-135):
+``x += mixer(norm(x))``, then ``x += ffn(norm(x))``; the residual stream ``x`` stays
+32-bit and the normalised copy has the activation type."""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from ..config.spec import BlockSpec
+from .base import BuildContext, ParamSpec, Part
+from .registry import build_feed_forward, build_mixer, build_norm, register_block
+
+
+class PreNormBlock(Part):
+    def __init__(self, spec: BlockSpec, ctx: BuildContext):
+        self.dtype = ctx.dtype
+        self.children = {"mixer_norm": build_norm(spec.mixer_norm, ctx),
+                         "mixer": build_mixer(spec.mixer, ctx),
+                         "ffn_norm": build_norm(spec.ffn_norm, ctx),
+                         "ffn": build_feed_forward(spec.ffn, ctx)}
+        self.mixer_norm = self.children["mixer_norm"]
+        self.mixer = self.children["mixer"]
+        self.ffn_norm = self.children["ffn_norm"]
+        self.ffn = self.children["ffn"]
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {f"{name}.{p}": spec for name, child in self.children.items()
+                for p, spec in child.param_specs().items()}
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        for name, child in self.children.items():
+            prefix = name + "."
+            child.bind({k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)})
+
+    def cache_request(self):
+        return self.mixer.cache_request()
+
+    def forward(self, step, x: torch.Tensor, cache, owns_cache: bool) -> None:
+        xn = step.workspace.get("block.xn", tuple(x.shape), self.dtype)
+        self.mixer_norm.forward(x, xn)
+        self.mixer.forward(step, xn, x, cache, owns_cache)
+        self.ffn_norm.forward(x, xn)
+        self.ffn.forward(step, xn, x)
+
+
+register_block("pre_norm", PreNormBlock)

@@ -1,0 +1,48 @@
+"""Dense gated feed-forward: ``y = down(act(gate(x)) * up(x))`` with no bias
+(rocml/src/forward/ffn.rs:36-107, rocml-kernels/kernels/silu_mul.hip:12-20).  Gate and up
+are one product over the concatenated weight; the residual sum is the down product's
+epilogue."""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from .. import ops
+from ..config.spec import GatedMlpSpec
+from ..errors import ConfigError
+from .base import BuildContext, FeedForward, ParamSpec
+from .registry import register_feed_forward
+
+
+class GatedMlp(FeedForward):
+    def __init__(self, spec: GatedMlpSpec, ctx: BuildContext):
+        if spec.activation != "silu":
+            raise ConfigError(f"activation {spec.activation!r} is not supported (silu only)")
+        self.spec = spec
+        self.dtype = ctx.dtype
+        self.w_gate_up: Optional[torch.Tensor] = None
+        self.w_down: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        s = self.spec
+        return {"gate_proj.weight": ParamSpec((s.intermediate, s.hidden)),
+                "up_proj.weight": ParamSpec((s.intermediate, s.hidden)),
+                "down_proj.weight": ParamSpec((s.hidden, s.intermediate))}
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.w_gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]], dim=0).contiguous()
+        self.w_down = tensors["down_proj.weight"]
+
+    def forward(self, step, xn, x_accum) -> None:
+        s = self.spec
+        n = step.n_tokens
+        ws = step.workspace
+        gate_up = ws.get("mlp.gate_up", (n, 2 * s.intermediate), torch.float32)
+        ops.gemm(xn, self.w_gate_up, gate_up, workspace=ws.scratch())
+        h = ws.get("mlp.h", (n, s.intermediate), self.dtype)
+        ops.swiglu(gate_up, h)
+        ops.gemm(h, self.w_down, x_accum, accumulate=True, workspace=ws.scratch())
+
+
+register_feed_forward("gated_mlp", GatedMlp)
