@@ -1,12 +1,89 @@
 // Matrix products of the decoder: out[M,N] (+)= X[M,K] * W[N,K]^T, weights row-major
-// [out, in] as the reference keeps them (rocml/src/weights/mod.rs:78-98).
+// [out, in] as the reference keeps them (rocml/src/weights/mod.rs:78-98).  bfloat16 operands
+// go to the MFMA kernels when their layout allows 16-byte loads; everything else, and the
+// whole 32-bit path, goes to the plain tiled kernel.
 #include "common.h"
 #include "gemm_tile.h"
+#include "gemm_mfma.h"
 
 ROCML_LAST_ERROR_FN(gemm)
 
-// algo: 0 = choose, 1 = plain tiled kernel.
+enum GemmAlgo : int { ALGO_AUTO = 0, ALGO_PLAIN = 1, ALGO_MFMA_TILE = 2, ALGO_MFMA_SKINNY = 3 };
+
+static int round_up(int a, int b) { return (a + b - 1) / b * b; }
+
+template <typename K>
+static int allow_lds(K kernel, int bytes, const char* name) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess)
+        return rocml_fail("%s: cannot reserve %d bytes of LDS: %s", name, bytes, hipGetErrorString(e));
+    return 0;
+}
+
+template <int EPI>
+static int launch_mfma_tile(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m,
+                            int n, int k, hipStream_t stream) {
+    static bool ready = false;
+    if (!ready) {
+        if (allow_lds(gemm_mfma_kernel<EPI>, GM_LDS_BYTES, "gemm")) return 1;
+        ready = true;
+    }
+    int tiles_m = ceil_div(m, GM_BM), tiles_n = ceil_div(n, GM_BN);
+    int n_tiles = tiles_m * tiles_n;
+    int grid = round_up(n_tiles, 8);
+    gemm_mfma_kernel<EPI><<<grid, GM_THREADS, GM_LDS_BYTES, stream>>>(
+        (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, tiles_m, n_tiles);
+    return 0;
+}
+
+template <int MT, int EPI>
+static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m, int n,
+                         int k, void* workspace, long long workspace_bytes, hipStream_t stream) {
+    constexpr int LDS = 2 * MT * 16 * GS_ROW * 16;
+    static bool ready = false;
+    if (!ready) {
+        if (allow_lds(gemm_skinny_kernel<MT, EPI, false>, LDS, "gemm")) return 1;
+        if (allow_lds(gemm_skinny_kernel<MT, EPI, true>, LDS, "gemm")) return 1;
+        ready = true;
+    }
+    int blocks_n = ceil_div(n, GS_BN);
+    int target = MT == 4 ? 256 : 512;
+    int splits = target / blocks_n;
+    int by_k = k / 512;
+    if (splits > by_k) splits = by_k;
+    if (splits > 16) splits = 16;
+    if (splits < 1) splits = 1;
+    long long per_split = (long long)m * n * sizeof(float);
+    if (splits > 1 && (long long)splits * per_split > workspace_bytes)
+        splits = workspace ? (int)(workspace_bytes / per_split) : 1;
+    if (splits < 1) splits = 1;
+    int k_per_split = round_up(ceil_div(k, splits), GS_KC);
+    splits = ceil_div(k, k_per_split);
+    dim3 grid(blocks_n, splits);
+    if (splits == 1) {
+        gemm_skinny_kernel<MT, EPI, false><<<grid, GS_THREADS, LDS, stream>>>(
+            (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
+    } else {
+        gemm_skinny_kernel<MT, EPI, true><<<grid, GS_THREADS, LDS, stream>>>(
+            (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, workspace, n, m, n, k, k_per_split);
+        long long total = (long long)m * n;
+        gemm_splitk_reduce_kernel<EPI><<<ceil_div(total, 256), 256, 0, stream>>>(
+            (const float*)workspace, out, ldo, m, n, splits);
+    }
+    return 0;
+}
+
+template <int EPI>
+static int launch_skinny_m(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m, int n,
+                           int k, void* workspace, long long workspace_bytes, hipStream_t stream) {
+    if (m <= 16) return launch_skinny<1, EPI>(x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, stream);
+    if (m <= 32) return launch_skinny<2, EPI>(x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, stream);
+    return launch_skinny<4, EPI>(x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, stream);
+}
+
+// algo: 0 = choose, 1 = plain tiled kernel, 2 = MFMA tile kernel, 3 = MFMA few-rows kernel.
 // accumulate: out += product (out must be 32-bit); this is the residual sum's epilogue.
+// workspace: device memory for split-K partial sums (may be null: no split).
 ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, int w_dtype, int ldw,
                             void* out, int out_dtype, int ldo, int m, int n, int k, int accumulate,
                             int algo, void* workspace, long long workspace_bytes,
@@ -15,16 +92,38 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
     ROCML_REQUIRE(ldx >= k && ldw >= k && ldo >= n, "gemm: row strides (%d, %d, %d) below (K, K, N)",
                   ldx, ldw, ldo);
     ROCML_REQUIRE(!accumulate || out_dtype == ROCML_F32, "gemm: accumulation needs a 32-bit output");
-    (void)algo; (void)workspace; (void)workspace_bytes;
+    ROCML_REQUIRE(algo >= ALGO_AUTO && algo <= ALGO_MFMA_SKINNY, "gemm: unknown algorithm %d", algo);
     if (m == 0) return 0;
-    if (x_dtype == ROCML_F32 && w_dtype == ROCML_F32 && out_dtype == ROCML_F32)
+    bool bf16_in = x_dtype == ROCML_BF16 && w_dtype == ROCML_BF16;
+    bool mfma_ok = bf16_in && k % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 &&
+                   ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
+    if (algo == ALGO_MFMA_TILE || algo == ALGO_MFMA_SKINNY)
+        ROCML_REQUIRE(mfma_ok, "gemm: the MFMA kernels need bfloat16 operands, K and row strides that are "
+                               "multiples of 8 and 16-byte aligned pointers (K=%d ldx=%d ldw=%d)", k, ldx, ldw);
+    if (algo == ALGO_MFMA_SKINNY)
+        ROCML_REQUIRE(m <= 64, "gemm: the few-rows kernel takes at most 64 rows, got %d", m);
+    int epi = accumulate ? EPI_ACC : (out_dtype == ROCML_BF16 ? EPI_BF16 : EPI_F32);
+    ROCML_REQUIRE(out_dtype == ROCML_F32 || out_dtype == ROCML_BF16, "gemm: unknown output type %d", out_dtype);
+    bool use_mfma = mfma_ok && algo != ALGO_PLAIN;
+    if (use_mfma) {
+        bool skinny = algo == ALGO_MFMA_SKINNY || (algo == ALGO_AUTO && m <= 64);
+        int rc;
+#define BY_EPI(fn, ...)                                              \
+        (epi == EPI_F32 ? fn<EPI_F32>(__VA_ARGS__)                   \
+         : epi == EPI_BF16 ? fn<EPI_BF16>(__VA_ARGS__) : fn<EPI_ACC>(__VA_ARGS__))
+        if (skinny) rc = BY_EPI(launch_skinny_m, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, stream);
+        else rc = BY_EPI(launch_mfma_tile, x, ldx, w, ldw, out, ldo, m, n, k, stream);
+#undef BY_EPI
+        if (rc) return rc;
+    } else if (x_dtype == ROCML_F32 && w_dtype == ROCML_F32 && out_dtype == ROCML_F32) {
         launch_gemm_tile<float, float, float>(x, ldx, w, ldw, out, ldo, m, n, k, accumulate, stream);
-    else if (x_dtype == ROCML_BF16 && w_dtype == ROCML_BF16 && out_dtype == ROCML_F32)
+    } else if (bf16_in && out_dtype == ROCML_F32) {
         launch_gemm_tile<bf16_t, bf16_t, float>(x, ldx, w, ldw, out, ldo, m, n, k, accumulate, stream);
-    else if (x_dtype == ROCML_BF16 && w_dtype == ROCML_BF16 && out_dtype == ROCML_BF16)
+    } else if (bf16_in && out_dtype == ROCML_BF16) {
         launch_gemm_tile<bf16_t, bf16_t, bf16_t>(x, ldx, w, ldw, out, ldo, m, n, k, 0, stream);
-    else
-        return rocml_fail("gemm: unsupported dtype triple x=%d w=%d out=%d", x_dtype, w_dtype, out_dtype);
+    } else {
+        return rocml_fail("gemm: unsupported type triple x=%d w=%d out=%d", x_dtype, w_dtype, out_dtype);
+    }
     ROCML_CHECK_LAUNCH("gemm");
     return 0;
 }

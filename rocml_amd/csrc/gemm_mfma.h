@@ -1,0 +1,255 @@
+// bfloat16 matrix products on the gfx950 matrix cores: out[M,N] (+)= X[M,K] * W[N,K]^T with
+// 32-bit accumulation.  Both operands are K-contiguous, which is what an MFMA lane wants: 8
+// consecutive K values (16 bytes) of one row.
+//
+// Two kernels:
+//  * gemm_mfma_kernel, many rows (prefill): 128x128 output tile per 256-thread block, four
+//    waves in 2x2, each wave 64x64 = 2x2 tiles of v_mfma_f32_32x32x16_bf16; K staged 64 at a
+//    time through double-buffered LDS with one barrier per stage; rows padded by 16 bytes so
+//    that 128-bit LDS reads of 16 rows fall into 16 different bank groups.  The idea of the
+//    tiling (big tile per block, 2x2 fragments per wave, padded double-buffered LDS) is the
+//    reference's WMMA kernel (rocml-kernels/kernels/gemm_xwt_wmma_impl.h:211-378); layouts and
+//    sizes are for wave64 MFMA.  Blocks are renumbered so that each of the 8 XCDs works on a
+//    contiguous range of tiles and its L2 sees few weight panels.
+//  * gemm_skinny_kernel, few rows (decode, M <= 64): memory-bound; a block owns 64 weight rows
+//    and a K range, each wave 16 rows.  Weights go straight from global memory into MFMA
+//    operand registers (v_mfma_f32_16x16x32_bf16), 8 loads of 16 bytes in flight per lane; the
+//    activations of the K range are shared through LDS.  Split-K partial sums go to a
+//    workspace and are added in split order by a second kernel, so results do not depend on
+//    timing (rocml-kernels/kernels/gemm_splitk_reduce.hip:4-10 has the same rule).
+#pragma once
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+__device__ __forceinline__ bf16x8_t as_frag(uint4 v) { return __builtin_bit_cast(bf16x8_t, v); }
+
+// Unconditional 16-byte load from an address the caller has clamped into range, zeroed
+// afterwards when the element is outside the matrix: a load under a branch would be waited for
+// before the next one is issued.
+__device__ __forceinline__ uint4 load16_or_zero(const bf16_t* p, bool ok) {
+    uint4 v = *(const uint4*)p;
+    v.x = ok ? v.x : 0u; v.y = ok ? v.y : 0u; v.z = ok ? v.z : 0u; v.w = ok ? v.w : 0u;
+    return v;
+}
+
+enum GemmEpilogue : int { EPI_F32 = 0, EPI_BF16 = 1, EPI_ACC = 2 };
+
+template <int EPI>
+__device__ __forceinline__ void epilogue_store(void* out, size_t idx, float v) {
+    if (EPI == EPI_F32) ((float*)out)[idx] = v;
+    else if (EPI == EPI_BF16) ((bf16_t*)out)[idx] = f32_to_bf16(v);
+    else ((float*)out)[idx] += v;
+}
+
+// ---- many rows ---------------------------------------------------------------------------
+constexpr int GM_BM = 128, GM_BN = 128, GM_BK = 64, GM_THREADS = 256;
+constexpr int GM_ROW = GM_BK / 8 + 1;                 // uint4 per LDS row, one of padding
+constexpr int GM_TILE = GM_BM * GM_ROW;               // uint4 per operand tile
+constexpr int GM_LDS_BYTES = 2 * 2 * GM_TILE * 16;    // two stages, two operands
+
+template <int EPI>
+__global__ void __launch_bounds__(GM_THREADS)
+gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw,
+                 void* __restrict__ out, int ldo, int m, int n, int k, int tiles_m, int n_tiles) {
+    extern __shared__ uint4 gm_smem[];
+    int per_xcd = gridDim.x / 8;
+    int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (logical >= n_tiles) return;
+    int m0 = (logical % tiles_m) * GM_BM, n0 = (logical / tiles_m) * GM_BN;
+    int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int wm = wave >> 1, wn = wave & 1;
+    int lrow = tid >> 3, lkc = tid & 7;
+    int nk = (k + GM_BK - 1) / GM_BK;
+    uint4 ra[4], rb[4];
+    f32x16_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    auto load_global = [&](int kt) {
+        int gk = kt * GM_BK + lkc * 8;
+        bool kin = gk < k;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int row = lrow + 32 * i;
+            bool oka = kin && (m0 + row) < m;
+            bool okb = kin && (n0 + row) < n;
+            ra[i] = load16_or_zero(x + (size_t)min(m0 + row, m - 1) * ldx + (kin ? gk : 0), oka);
+            rb[i] = load16_or_zero(w + (size_t)min(n0 + row, n - 1) * ldw + (kin ? gk : 0), okb);
+        }
+    };
+    auto store_lds = [&](int buf) {
+        uint4* sa = gm_smem + buf * 2 * GM_TILE;
+        uint4* sb = sa + GM_TILE;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int row = lrow + 32 * i;
+            sa[row * GM_ROW + lkc] = ra[i];
+            sb[row * GM_ROW + lkc] = rb[i];
+        }
+    };
+
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+        int buf = kt & 1;
+        bool more = kt + 1 < nk;
+        if (more) load_global(kt + 1);
+        const uint4* sa = gm_smem + buf * 2 * GM_TILE;
+        const uint4* sb = sa + GM_TILE;
+#pragma unroll
+        for (int kk = 0; kk < GM_BK / 16; ++kk) {
+            bf16x8_t a[2], b[2];
+            int col = kk * 2 + (lane >> 5);
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                a[i] = as_frag(sa[(wm * 64 + i * 32 + (lane & 31)) * GM_ROW + col]);
+                b[i] = as_frag(sb[(wn * 64 + i * 32 + (lane & 31)) * GM_ROW + col]);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) store_lds(buf ^ 1);
+        __syncthreads();
+    }
+    // Accumulator element e of a lane: row 8*(e/4) + 4*(lane/32) + e%4, column lane%32.
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            int gn = n0 + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                int gm = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                if (gm < m && gn < n) epilogue_store<EPI>(out, (size_t)gm * ldo + gn, acc[i][j][e]);
+            }
+        }
+}
+
+// ---- few rows ----------------------------------------------------------------------------
+constexpr int GS_BN = 64, GS_KC = 256, GS_THREADS = 256;
+constexpr int GS_ROW = GS_KC / 8 + 1;                 // uint4 per LDS row of activations
+
+// PARTIAL: write 32-bit partial sums [split][M][N] instead of the epilogue.
+template <int MT, int EPI, bool PARTIAL>
+__global__ void __launch_bounds__(GS_THREADS)
+gemm_skinny_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw,
+                   void* __restrict__ out, int ldo, int m, int n, int k, int k_per_split) {
+    extern __shared__ uint4 gs_smem[];                // [2][MT*16][GS_ROW]
+    constexpr int ROWS = MT * 16;
+    constexpr int XCHUNKS = ROWS * (GS_KC / 8) / GS_THREADS;   // 16-byte pieces per thread
+    int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int n0 = blockIdx.x * GS_BN + wave * 16;
+    int ks = blockIdx.y * k_per_split;
+    int ke = min(k, ks + k_per_split);
+    int n_chunks = (ke - ks + GS_KC - 1) / GS_KC;
+    int wrow = n0 + (lane & 15);
+    bool wok = wrow < n;
+    const bf16_t* wbase = w + (size_t)(wok ? wrow : 0) * ldw + (lane >> 4) * 8;
+    uint4 wcur[8], wnext[8], xr[XCHUNKS];
+    f32x4_t acc[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    // Blocks start their K loop at different chunks and wrap around: row strides are often a
+    // power of two, and blocks that all read the same K window at once would queue up on a few
+    // memory channels.
+    int rot = (blockIdx.x * 5 + blockIdx.y * 3) % n_chunks;
+    auto chunk_base = [&](int c) {
+        int cc = c + rot;
+        if (cc >= n_chunks) cc -= n_chunks;
+        return ks + cc * GS_KC;
+    };
+    auto load_w = [&](int c, uint4* dst) {
+        int kb = chunk_base(c);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            int gk = kb + j * 32 + (lane >> 4) * 8;
+            bool ok = gk < ke;
+            dst[j] = load16_or_zero(ok ? wbase + kb + j * 32 : w, wok && ok);
+        }
+    };
+    auto load_x = [&](int c) {
+        int kb = chunk_base(c);
+#pragma unroll
+        for (int i = 0; i < XCHUNKS; ++i) {
+            int piece = tid + i * GS_THREADS;
+            int row = piece / (GS_KC / 8), kc = piece % (GS_KC / 8);
+            int gk = kb + kc * 8;
+            bool ok = gk < ke;
+            xr[i] = load16_or_zero(ok ? x + (size_t)min(row, m - 1) * ldx + gk : x, ok && row < m);
+        }
+    };
+    auto store_x = [&](int buf) {
+        uint4* sx = gs_smem + buf * ROWS * GS_ROW;
+#pragma unroll
+        for (int i = 0; i < XCHUNKS; ++i) {
+            int piece = tid + i * GS_THREADS;
+            sx[(piece / (GS_KC / 8)) * GS_ROW + piece % (GS_KC / 8)] = xr[i];
+        }
+    };
+
+    load_w(0, wcur);
+    load_x(0);
+    store_x(0);
+    __syncthreads();
+    for (int c = 0; c < n_chunks; ++c) {
+        int buf = c & 1;
+        bool more = c + 1 < n_chunks;
+        if (more) {
+            load_w(c + 1, wnext);
+            load_x(c + 1);
+        }
+        const uint4* sx = gs_smem + buf * ROWS * GS_ROW;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            bf16x8_t a = as_frag(wcur[j]);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                bf16x8_t b = as_frag(sx[(mt * 16 + (lane & 15)) * GS_ROW + j * 4 + (lane >> 4)]);
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
+            }
+        }
+        if (more) {
+            store_x(buf ^ 1);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) wcur[j] = wnext[j];
+        }
+        __syncthreads();
+    }
+    // Accumulator element e of a lane: weight row (lane/16)*4 + e, activation row lane%16.
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        int gm = mt * 16 + (lane & 15);
+        if (gm >= m) continue;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            int gn = n0 + (lane >> 4) * 4 + e;
+            if (gn >= n) continue;
+            if (PARTIAL) ((float*)out)[((size_t)blockIdx.y * m + gm) * n + gn] = acc[mt][e];
+            else epilogue_store<EPI>(out, (size_t)gm * ldo + gn, acc[mt][e]);
+        }
+    }
+}
+
+// out[m][n] (+)= sum over splits, in split order.
+template <int EPI>
+__global__ void gemm_splitk_reduce_kernel(const float* __restrict__ partial, void* __restrict__ out,
+                                          int ldo, int m, int n, int splits) {
+    long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (long long)m * n) return;
+    int gm = (int)(idx / n), gn = (int)(idx - (long long)gm * n);
+    float s = 0.f;
+    for (int i = 0; i < splits; ++i) s += partial[(size_t)i * m * n + idx];
+    epilogue_store<EPI>(out, (size_t)gm * ldo + gn, s);
+}

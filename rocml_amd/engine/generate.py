@@ -1,0 +1,190 @@
+"""The generation loop: batches of unequal prompts, stop tokens, sequences that end
+earlier, and as many batches one after another as there are requests.
+
+Per sequence the flow is the reference's (rocml/src/generate/resumed.rs:193-233): the
+prompt in one step, then sample, stop on a stop token without emitting it, emit, and run
+the token.  Around it, which the reference does not have: requests are taken in order
+into a batch while slots and cache pages for their prompt and their whole output are
+free; the batch starts together; a sequence that ends leaves the batch and gives its
+slot back; when the batch is empty the next one starts.  The loop decides on token ids
+only and talks to the model through a small backend, so its decisions can be tested
+without a GPU.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import FrozenSet, List, Optional, Sequence
+
+from ..errors import CacheFullError, RocmlError
+from ..sampling.params import SamplingParams
+from ..sampling.sampler import SequenceSampling
+
+
+@dataclass
+class Request:
+    prompt: Sequence[int]
+    max_new_tokens: int = 64
+    params: SamplingParams = field(default_factory=SamplingParams)
+    stop_tokens: FrozenSet[int] = frozenset()
+
+
+@dataclass
+class Result:
+    tokens: List[int]
+    finish_reason: str            # "stop", "length", "context" or "empty"
+    prompt_tokens: int
+
+
+@dataclass
+class GenerateStats:
+    """Token counts and seconds of the two phases (rocml/src/generate/mod.rs:27-51)."""
+    prompt_tokens: int = 0
+    generated_tokens: int = 0
+    prompt_seconds: float = 0.0
+    decode_seconds: float = 0.0
+    batches: int = 0
+    decode_steps: int = 0
+
+    def prompt_tok_s(self) -> float:
+        return self.prompt_tokens / self.prompt_seconds if self.prompt_seconds > 0 else 0.0
+
+    def decode_tok_s(self) -> float:
+        return self.generated_tokens / self.decode_seconds if self.decode_seconds > 0 else 0.0
+
+
+class EngineBackend:
+    """The loop's view of the engine and the sampler."""
+
+    def __init__(self, engine, sampler=None):
+        from ..sampling.sampler import DeviceSampler
+        self.engine = engine
+        self.sampler = sampler or DeviceSampler(engine.model.device)
+        self.max_positions = engine.model.spec.max_positions
+
+    def can_admit(self, lengths: Sequence[int]) -> bool:
+        """Whether sequences that will grow to ``lengths`` fit beside nothing else."""
+        cache = self.engine.cache
+        if len(lengths) > cache.slots.n_free:
+            return False
+        from ..cache import pages_for
+        for g in cache.kv_groups:
+            if sum(pages_for(n, g.page_size) for n in lengths) > g.n_free_pages:
+                return False
+        return True
+
+    def new_sequence(self) -> int:
+        return self.engine.new_sequence()
+
+    def release(self, slot: int) -> None:
+        self.engine.release(slot)
+
+    def step(self, slots: Sequence[int], tokens: Sequence[Sequence[int]]):
+        from .batch import StepEntry
+        return self.engine.step([StepEntry(s, list(t), [len(t) - 1]) for s, t in zip(slots, tokens)])
+
+    def sample(self, logits, seqs: Sequence[SequenceSampling]) -> List[int]:
+        return self.sampler.sample(logits, seqs)
+
+    def synchronize(self) -> None:
+        import torch
+        torch.cuda.synchronize()
+
+
+@dataclass
+class _Live:
+    index: int
+    request: Request
+    slot: int
+    sampling: SequenceSampling
+    out: List[int] = field(default_factory=list)
+
+
+class Generator:
+    def __init__(self, backend, max_batch: int = 64):
+        if max_batch < 1:
+            raise RocmlError("max_batch must be at least 1")
+        self.backend = backend
+        self.max_batch = max_batch
+        self.stats = GenerateStats()
+
+    def _final_length(self, r: Request) -> int:
+        return min(len(r.prompt) + r.max_new_tokens, self.backend.max_positions)
+
+    def _take_batch(self, requests: Sequence[Request], first: int) -> int:
+        """Number of requests, from ``first`` on, that start together."""
+        lengths: List[int] = []
+        n = 0
+        while first + n < len(requests) and n < self.max_batch:
+            r = requests[first + n]
+            if len(r.prompt) == 0:
+                if n == 0:
+                    return 0      # handled alone by the caller
+                break
+            if len(r.prompt) > self.backend.max_positions:
+                raise RocmlError(f"request {first + n}: a prompt of {len(r.prompt)} tokens exceeds the "
+                                 f"model's {self.backend.max_positions} positions")
+            if not self.backend.can_admit(lengths + [self._final_length(r)]):
+                break
+            lengths.append(self._final_length(r))
+            n += 1
+        if n == 0:
+            raise CacheFullError(f"request {first} does not fit the cache even alone "
+                                 f"({self._final_length(requests[first])} positions)")
+        return n
+
+    def run(self, requests: Sequence[Request]) -> List[Result]:
+        results: List[Optional[Result]] = [None] * len(requests)
+        at = 0
+        while at < len(requests):
+            n = self._take_batch(requests, at)
+            if n == 0:
+                # An empty prompt gives no logits and so no token
+                # (rocml/src/forward/chunk_forward.rs:38-40, rocml/src/generate/resumed.rs:215).
+                results[at] = Result([], "empty", 0)
+                at += 1
+                continue
+            self._run_batch(requests, at, n, results)
+            at += n
+        return results  # type: ignore[return-value]
+
+    def _run_batch(self, requests, first: int, n: int, results) -> None:
+        be = self.backend
+        live = [_Live(first + i, requests[first + i], be.new_sequence(),
+                      SequenceSampling.start(requests[first + i].params, first + i, requests[first + i].prompt))
+                for i in range(n)]
+        self.stats.batches += 1
+        t0 = time.perf_counter()
+        logits = be.step([s.slot for s in live], [list(s.request.prompt) for s in live])
+        be.synchronize()
+        t1 = time.perf_counter()
+        self.stats.prompt_seconds += t1 - t0
+        self.stats.prompt_tokens += sum(len(s.request.prompt) for s in live)
+        while live:
+            drawn = be.sample(logits, [s.sampling for s in live])
+            still: List[_Live] = []
+            for s, tok in zip(live, drawn):
+                reason = None
+                if s.request.max_new_tokens <= 0:
+                    reason = "length"
+                elif tok in s.request.stop_tokens:
+                    reason = "stop"          # not emitted (rocml/src/generate/resumed.rs:217-219)
+                else:
+                    s.out.append(tok)
+                    s.sampling.history.append(tok)
+                    self.stats.generated_tokens += 1
+                    if len(s.out) >= s.request.max_new_tokens:
+                        reason = "length"
+                    elif len(s.request.prompt) + len(s.out) >= be.max_positions:
+                        reason = "context"
+                if reason is None:
+                    still.append(s)
+                else:
+                    results[s.index] = Result(s.out, reason, len(s.request.prompt))
+                    be.release(s.slot)
+            live = still
+            if live:
+                logits = be.step([s.slot for s in live], [[s.out[-1]] for s in live])
+                self.stats.decode_steps += 1
+        be.synchronize()
+        self.stats.decode_seconds += time.perf_counter() - t1

@@ -1,0 +1,79 @@
+"""Draws the next token of every sequence of a batch on the device.
+
+The order of operations is the reference's host sampler (rocml/src/sample.rs:90-166):
+repeat penalty over the last ``repeat_penalty_window`` tokens of prompt and output,
+greedy when the temperature is not positive, else temperature, top-k, softmax, top-p and
+a draw with one uniform number from the sequence's own xorshift64* stream
+(rocml/src/sample.rs:56-83).  Logits stay on the device; only the drawn ids come back.
+Where candidates tie exactly at the k-th value the lowest ids are kept, top-p keeps all
+tokens as probable as the last one it needs, and the draw walks the vocabulary in id
+order (the reference walks it in order of probability): the distribution is the same,
+the token drawn for a given uniform number may differ.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from .. import ops
+from .params import Rng, SamplingParams, sequence_seed
+
+
+@dataclass
+class SequenceSampling:
+    """Sampling state of one sequence: its parameters, random stream and history."""
+    params: SamplingParams
+    rng: Rng
+    history: List[int] = field(default_factory=list)
+
+    @staticmethod
+    def start(params: SamplingParams, index: int, prompt: Sequence[int]) -> "SequenceSampling":
+        return SequenceSampling(params, Rng(sequence_seed(params.seed, index)), list(prompt))
+
+
+class DeviceSampler:
+    def __init__(self, device):
+        self.device = torch.device(device)
+        self._work: Optional[torch.Tensor] = None
+
+    def sample(self, logits: torch.Tensor, seqs: Sequence[SequenceSampling]) -> List[int]:
+        """``logits`` is ``[B, V]`` 32-bit on the device, row ``b`` for ``seqs[b]``.  Returns
+        the drawn ids and appends them to nothing: the caller decides what a token means."""
+        batch, vocab = logits.shape
+        assert batch == len(seqs)
+        out = torch.empty(batch, dtype=torch.int32, device=self.device)
+        if all(s.params.is_greedy() and not s.params.penalty_active() for s in seqs):
+            ops.argmax(logits, out)
+            return out.cpu().tolist()
+        if self._work is None or self._work.numel() < logits.numel():
+            self._work = torch.empty(logits.numel(), dtype=torch.float32, device=self.device)
+        temperature = np.zeros(batch, np.float32)
+        uniform = np.zeros(batch, np.float32)
+        top_k = np.zeros(batch, np.int32)
+        top_p = np.full(batch, -1.0, np.float32)
+        penalty = np.zeros(batch, np.float32)
+        window = max([s.params.repeat_penalty_window for s in seqs if s.params.penalty_active()] + [1])
+        hist = np.zeros((batch, window), np.int32)
+        hist_len = np.zeros(batch, np.int32)
+        for b, s in enumerate(seqs):
+            p = s.params
+            if p.penalty_active():
+                recent = s.history[-p.repeat_penalty_window:] if p.repeat_penalty_window > 0 else []
+                penalty[b] = p.repeat_penalty
+                hist[b, :len(recent)] = recent
+                hist_len[b] = len(recent)
+            if p.is_greedy():
+                continue
+            temperature[b] = p.temperature
+            top_k[b] = 0 if p.top_k is None else max(1, int(p.top_k))
+            top_p[b] = -1.0 if p.top_p is None else min(max(float(p.top_p), 0.0), 1.0)
+            uniform[b] = s.rng.next_f32()
+        floats = torch.from_numpy(np.stack([temperature, uniform, top_p, penalty])).to(self.device)
+        ints = torch.from_numpy(np.concatenate([top_k, hist_len, hist.reshape(-1)])).to(self.device)
+        ops.sample(logits, self._work, floats[0], floats[1], out, top_k=ints[:batch], top_p=floats[2],
+                   penalty=floats[3], history=ints[2 * batch:].view(batch, window),
+                   history_len=ints[batch:2 * batch])
+        return out.cpu().tolist()

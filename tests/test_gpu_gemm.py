@@ -1,0 +1,79 @@
+"""The matrix product kernels alone against a plain 32-bit product of the same operands,
+at sizes other than the engine's: sizes that are no multiple of a tile, single rows,
+every algorithm and epilogue."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from rocml_amd import ops  # noqa: E402
+
+PLAIN, TILE, SKINNY = 1, 2, 3
+
+
+def _operands(m, n, k, dtype, seed):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    x = torch.randn(m, k, generator=g).to(dtype).cuda()
+    w = (torch.randn(n, k, generator=g) * 0.05).to(dtype).cuda()
+    return x, w
+
+
+def _ref(x, w):
+    return (x.double() @ w.double().t())
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 7, 5), (3, 64, 16), (65, 130, 33), (200, 96, 257), (17, 384, 96)])
+def test_plain_float32(m, n, k):
+    x, w = _operands(m, n, k, torch.float32, 1)
+    out = torch.empty(m, n, dtype=torch.float32, device="cuda")
+    ops.gemm(x, w, out, algo=PLAIN)
+    ref = _ref(x, w)
+    assert float((out.double() - ref).abs().max()) < 1e-5 * max(1.0, float(ref.abs().max()))
+    base = torch.randn(m, n, device="cuda")
+    acc = base.clone()
+    ops.gemm(x, w, acc, accumulate=True, algo=PLAIN)
+    assert float((acc.double() - (ref + base.double())).abs().max()) < 1e-5 * max(1.0, float(ref.abs().max()))
+
+
+SHAPES = [(1, 64, 64), (5, 200, 72), (16, 130, 512), (17, 96, 264), (33, 4096, 1024), (64, 257, 4096),
+          (8, 1000, 2056), (128, 128, 64), (129, 300, 200), (300, 515, 72), (2048, 512, 1024)]
+
+
+@pytest.mark.parametrize("algo", [PLAIN, TILE, SKINNY])
+@pytest.mark.parametrize("m,n,k", SHAPES)
+def test_bfloat16_algorithms(m, n, k, algo):
+    if algo == SKINNY and m > 64:
+        pytest.skip("the few-rows kernel takes at most 64 rows")
+    x, w = _operands(m, n, k, torch.bfloat16, 2)
+    ref = _ref(x, w)
+    scale = max(1.0, float(ref.abs().max()))
+    ws = torch.empty(64 << 20, dtype=torch.uint8, device="cuda")
+    out = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
+    ops.gemm(x, w, out, algo=algo, workspace=ws)
+    assert float((out.double() - ref).abs().max()) < 2e-5 * scale, "32-bit output"
+    out16 = torch.empty(m, n, dtype=torch.bfloat16, device="cuda")
+    ops.gemm(x, w, out16, algo=algo, workspace=ws)
+    assert float((out16.double() - ref).abs().max()) < 5e-3 * scale, "bfloat16 output"
+    base = torch.randn(m, n, device="cuda")
+    acc = base.clone()
+    ops.gemm(x, w, acc, accumulate=True, algo=algo, workspace=ws)
+    assert float((acc.double() - (ref + base.double())).abs().max()) < 2e-5 * scale, "accumulating"
+
+
+def test_strided_rows_and_refusals():
+    from rocml_amd.errors import KernelError
+    big = torch.randn(40, 200, device="cuda").to(torch.bfloat16)
+    x = big[:, 8:72]                       # row stride 200, 64 columns
+    w = (torch.randn(48, 64, device="cuda") * 0.1).to(torch.bfloat16)
+    out = torch.empty(40, 48, dtype=torch.float32, device="cuda")
+    ops.gemm(x, w, out)
+    assert float((out.double() - _ref(x, w)).abs().max()) < 1e-4
+    odd = torch.randn(4, 36, device="cuda").to(torch.bfloat16)   # K = 36 is no multiple of 8
+    w2 = torch.randn(8, 36, device="cuda").to(torch.bfloat16)
+    out2 = torch.empty(4, 8, dtype=torch.float32, device="cuda")
+    ops.gemm(odd, w2, out2)                # falls back to the plain kernel
+    assert float((out2.double() - _ref(odd, w2)).abs().max()) < 1e-3
+    with pytest.raises(KernelError):
+        ops.gemm(odd, w2, out2, algo=TILE)
+    with pytest.raises(KernelError):
+        ops.gemm(x.cpu(), w, out)
