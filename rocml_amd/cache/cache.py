@@ -11,9 +11,9 @@ are kept here, for many sequences:
 * a **slot** stands for one live sequence and knows its length;
 * cache lines (one per execution of a layer that owns a cache) with the same needs form
   a **group** with storage of its own.  A key/value group is a pool of pages of
-  ``page_size`` positions, laid out ``[line, page, Hkv, page_size, D]`` so that one
-  head's positions of a page are contiguous; each slot maps its logical pages to pool
-  pages.  A group with a window gives pages back as soon as no later query can see them;
+  ``page_size`` positions, keys laid out ``[line, page, Hkv, page_size, D]`` and values
+  ``[line, page, Hkv, D, page_size]``, so that one head's part of a page is contiguous;
+  each slot maps its logical pages to pool pages.  A group with a window gives pages back as soon as no later query can see them;
 * a **state group** is ``[line, slot, *shape]`` and a slot's part is zeroed when the
   slot is handed out;
 * pages are not cleared when a slot is freed or handed out again.
@@ -84,9 +84,12 @@ class KVGroup:
         self.n_lines = n_lines
         self.n_pages = n_pages
         self.page_size = page_size
-        shape = (n_lines, n_pages, request.n_kv_heads, page_size, request.head_dim)
-        self.k = torch.empty(shape, dtype=dtype, device=device)
-        self.v = torch.empty(shape, dtype=dtype, device=device)
+        # Values are transposed inside a page, which is the order the attention kernels
+        # multiply them in.  Zeroed once: rows beyond a sequence's length are never counted,
+        # but they are multiplied by a zero weight and so must stay finite.
+        h, d = request.n_kv_heads, request.head_dim
+        self.k = torch.zeros((n_lines, n_pages, h, page_size, d), dtype=dtype, device=device)
+        self.v = torch.zeros((n_lines, n_pages, h, d, page_size), dtype=dtype, device=device)
         self._free = list(range(n_pages - 1, -1, -1))
         self._pages: Dict[int, List[int]] = {}   # slot -> logical page -> pool page, -1 once released
 
@@ -163,7 +166,7 @@ class CacheLineView:
     group: object
     line: int
     k: Optional[torch.Tensor] = None            # [pages, Hkv, page_size, D]
-    v: Optional[torch.Tensor] = None
+    v: Optional[torch.Tensor] = None            # [pages, Hkv, D, page_size]
     block_table: Optional[torch.Tensor] = None  # [B, width] int32 on the device, per step
     state: Optional[torch.Tensor] = None        # [slots, *shape]
     slots: Optional[torch.Tensor] = None        # [B] int32 on the device, per step

@@ -1,18 +1,102 @@
 // Attention over the paged key/value cache for gfx950.  One entry point for any step: the
 // query tokens of a step carry their sequence and position, keys and values are read from
 // the cache (the step's own keys were appended before), so prefill, decode and any cut of a
-// prompt run the same code.
+// prompt run the same code.  bfloat16 with a head size that is a multiple of 32 runs on the
+// matrix cores; everything else, and the whole 32-bit path, runs the plain kernel.
 #include "common.h"
 #include "attention_generic.h"
+#include "attention_mfma.h"
 
 ROCML_LAST_ERROR_FN(attention)
 
-// algo: 0 = choose, 1 = plain kernel.
+enum AttnAlgo : int { ATTN_AUTO = 0, ATTN_PLAIN = 1, ATTN_MFMA = 2 };
+
+static const float LOG2E = 1.4426950408889634f;
+
+template <typename K>
+static int allow_lds(K kernel, int bytes) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess)
+        return rocml_fail("attention: cannot reserve %d bytes of LDS: %s", bytes, hipGetErrorString(e));
+    return 0;
+}
+
+struct AttnArgs {
+    const bf16_t* q; bf16_t* out; const bf16_t* kcache; const bf16_t* vcache;
+    const int* block_table; int bt_width; const int* token_seq; const int* token_pos;
+    const int* cu_seqlens; int n_seqs; int n_tokens; int total_q_tiles; int max_len;
+    int hq, hkv; float scale; int window; void* workspace; long long workspace_bytes;
+    int n_splits_hint;
+};
+
+template <int D>
+static int launch_decode(const AttnArgs& a, hipStream_t stream) {
+    int group = a.hq / a.hkv;
+    int lds = 4 * group * (D + 4) * (int)sizeof(float);
+    static int allowed = 0;
+    if (lds > allowed) {
+        if (allow_lds(attn_decode_mfma_kernel<D>, lds)) return 1;
+        allowed = lds;
+    }
+    // Enough blocks to fill the chip, at most one split per page of the longest sequence.
+    int n_splits = a.n_splits_hint;
+    if (n_splits <= 0) {
+        n_splits = 512 / (a.n_tokens * a.hkv);
+        int max_pages = (a.max_len + AM_PAGE - 1) / AM_PAGE;
+        if (n_splits > max_pages) n_splits = max_pages;
+    }
+    if (n_splits > 64) n_splits = 64;
+    if (n_splits < 1) n_splits = 1;
+    long long per_split = (long long)a.n_tokens * a.hq * (D + 2) * sizeof(float);
+    if (n_splits > 1 && per_split * n_splits > a.workspace_bytes)
+        n_splits = a.workspace ? (int)(a.workspace_bytes / per_split) : 1;
+    if (n_splits < 1) n_splits = 1;
+    float* part_o = (float*)a.workspace;
+    float* part_ml = part_o ? part_o + (size_t)a.n_tokens * a.hq * n_splits * D : nullptr;
+    dim3 grid(n_splits, a.hkv, a.n_tokens);
+    attn_decode_mfma_kernel<D><<<grid, AM_THREADS, lds, stream>>>(
+        a.q, a.out, a.kcache, a.vcache, a.block_table, a.bt_width, a.token_seq, a.token_pos, a.hq, a.hkv,
+        a.scale * LOG2E, a.window, n_splits, part_o, part_ml);
+    if (n_splits > 1)
+        attn_decode_reduce_kernel<D><<<a.n_tokens * a.hq, D < 64 ? 64 : D, 0, stream>>>(part_o, part_ml, a.out, n_splits);
+    return 0;
+}
+
+template <int D>
+static int launch_prefill(const AttnArgs& a, hipStream_t stream) {
+    static bool ready = false;
+    if (!ready) {
+        if (allow_lds(attn_prefill_mfma_kernel<D>, PrefillLds<D>::BYTES)) return 1;
+        ready = true;
+    }
+    dim3 grid(a.total_q_tiles, a.hq);
+    attn_prefill_mfma_kernel<D><<<grid, AM_THREADS, PrefillLds<D>::BYTES, stream>>>(
+        a.q, a.out, a.kcache, a.vcache, a.block_table, a.bt_width, a.cu_seqlens, a.n_seqs, a.token_pos,
+        a.hq, a.hkv, a.scale * LOG2E, a.window);
+    return 0;
+}
+
+static bool mfma_head_dim(int d) { return d == 32 || d == 64 || d == 96 || d == 128 || d == 192 || d == 256; }
+
+#define BY_HEAD_DIM(fn, d, ...)                       \
+    ((d) == 32 ? fn<32>(__VA_ARGS__)                  \
+     : (d) == 64 ? fn<64>(__VA_ARGS__)                \
+     : (d) == 96 ? fn<96>(__VA_ARGS__)                \
+     : (d) == 128 ? fn<128>(__VA_ARGS__)              \
+     : (d) == 192 ? fn<192>(__VA_ARGS__) : fn<256>(__VA_ARGS__))
+
+// algo: 0 = choose, 1 = plain kernel, 2 = MFMA kernels (error if they cannot take the shapes).
+// cu_seqlens [n_seqs + 1] gives where each sequence's query tokens start (tokens of a sequence
+// are consecutive and in position order); max_new is the most query tokens of any sequence,
+// total_q_tiles the sum over sequences of ceil(tokens / 128), max_len the longest context.
+// workspace holds the partial results of split decode attention.
 ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, const void* vcache,
                                  int dtype, const int* block_table, int bt_width,
                                  const int* token_seq, const int* token_pos, int n_tokens, int hq,
                                  int hkv, int d, int page_size, float scale, int window, int algo,
-                                 void* workspace, long long workspace_bytes, hipStream_t stream) {
+                                 const int* cu_seqlens, int n_seqs, int max_new, int total_q_tiles,
+                                 int max_len, int n_splits, void* workspace, long long workspace_bytes,
+                                 hipStream_t stream) {
     ROCML_REQUIRE(n_tokens >= 0 && hq > 0 && hkv > 0 && d > 0 && page_size > 0 && bt_width > 0,
                   "attention: bad sizes T=%d Hq=%d Hkv=%d D=%d page=%d width=%d", n_tokens, hq, hkv,
                   d, page_size, bt_width);
@@ -20,8 +104,24 @@ ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, c
     ROCML_REQUIRE(window >= 0, "attention: negative window %d", window);
     ROCML_REQUIRE(d <= AG_BLOCK * AG_MAX_D_PER_THREAD, "attention: head_dim %d exceeds %d", d,
                   AG_BLOCK * AG_MAX_D_PER_THREAD);
-    (void)algo; (void)workspace; (void)workspace_bytes;
+    ROCML_REQUIRE(algo >= ATTN_AUTO && algo <= ATTN_MFMA, "attention: unknown algorithm %d", algo);
     if (n_tokens == 0) return 0;
+    bool decode = max_new == 1;
+    bool mfma_ok = dtype == ROCML_BF16 && page_size == AM_PAGE && mfma_head_dim(d) && max_new >= 1 &&
+                   (decode ? hq / hkv <= 16 : (cu_seqlens != nullptr && n_seqs > 0 && total_q_tiles > 0));
+    if (algo == ATTN_MFMA)
+        ROCML_REQUIRE(mfma_ok, "attention: the MFMA kernels need bfloat16, pages of 64 positions, a head size "
+                               "of 32, 64, 96, 128, 192 or 256, at most 16 query heads per kv head in decode and "
+                               "the sequence offsets in prefill (D=%d page=%d group=%d)", d, page_size, hq / hkv);
+    if (mfma_ok && algo != ATTN_PLAIN) {
+        AttnArgs a{(const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table,
+                   bt_width, token_seq, token_pos, cu_seqlens, n_seqs, n_tokens, total_q_tiles, max_len, hq, hkv,
+                   scale, window, workspace, workspace_bytes, n_splits};
+        int rc = decode ? BY_HEAD_DIM(launch_decode, d, a, stream) : BY_HEAD_DIM(launch_prefill, d, a, stream);
+        if (rc) return rc;
+        ROCML_CHECK_LAUNCH("attention");
+        return 0;
+    }
     dim3 grid(n_tokens, hq);
     size_t lds = (size_t)(d + AG_BLOCK) * sizeof(float);
     if (dtype == ROCML_F32)

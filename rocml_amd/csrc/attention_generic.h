@@ -5,6 +5,7 @@
 // scale, running maximum m, l = l * e^(m - m') + sum e^(s - m'), acc likewise, out = acc / l.
 // A query at position p sees keys [lo, p], lo = 0 or p - window + 1.  Keys are taken 256 at a
 // time: every thread scores one key, then the threads split the head's values.
+// Cache layout: keys [page, Hkv, page_size, D], values transposed in a page [page, Hkv, D, page_size].
 #pragma once
 #include "common.h"
 
@@ -77,8 +78,8 @@ attn_generic_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __res
             for (int jj = 0; jj < n_keys; ++jj) {
                 int key = c0 + jj;
                 int page = pages[key / page_size];
-                const T* vrow = vcache + (((size_t)page * hkv + kvh) * page_size + key % page_size) * d;
-                a = fmaf(ps[jj], Elem<T>::load(vrow + e), a);
+                const T* vcol = vcache + ((size_t)page * hkv + kvh) * d * page_size + key % page_size;
+                a = fmaf(ps[jj], Elem<T>::load(vcol + (size_t)e * page_size), a);
             }
             acc[r] = a;
         }

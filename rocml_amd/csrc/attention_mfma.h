@@ -1,0 +1,350 @@
+// bfloat16 attention over the paged cache on the gfx950 matrix cores.
+//
+// Cache layout (page_size = 64): keys [page, Hkv, 64, D], values transposed inside a page
+// [page, Hkv, D, 64].  With this layout both products read 8 or 4 consecutive elements per
+// lane: S^T = K * Q^T takes K rows along D, O^T = V^T * P^T takes V^T rows along the keys.
+// Both kernels compute the transposed products so that one lane owns one query column: the
+// running maximum, the sum and the rescaling of the output are lane-local and P^T is already
+// the MFMA operand for the second product (no shuffles, no LDS round trip for P).
+//
+// The algebra is the reference's online softmax (rocml-kernels/kernels/attn_decode.hip:151-170,
+// 227-254; attn_prefill_flash_impl.h:46-159): per query m' = max(m, s), acc and l scaled by
+// e^(m - m'), splits merged by log-sum-exp in split order.  Scores are scaled after the dot
+// product; exponentials are base 2 with log2(e) folded into the scale.
+#pragma once
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+constexpr int AM_PAGE = 64;
+constexpr int AM_THREADS = 256;
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+    return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+}
+
+// ---- decode: one query token per sequence ----------------------------------------------------
+// grid (n_splits, Hkv, tokens), 4 waves; the block's pages are cut into 32-key pieces that the
+// waves take in turn; all query heads of the kv head ride in the 16 columns of the MFMA.
+template <int D>
+__global__ void __launch_bounds__(AM_THREADS)
+attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
+                        const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
+                        const int* __restrict__ block_table, int bt_width,
+                        const int* __restrict__ token_seq, const int* __restrict__ token_pos, int hq,
+                        int hkv, float scale_log2e, int window, int n_splits,
+                        float* __restrict__ part_o, float* __restrict__ part_ml) {
+    constexpr int KD = D / 32;      // MFMA steps along D for the scores
+    constexpr int DT = D / 16;      // 16-row tiles of the output
+    extern __shared__ float sm_o[];                 // [4 waves][group][D + 4]
+    __shared__ float sm_m[4][16], sm_l[4][16];
+    int split = blockIdx.x, kvh = blockIdx.y, t = blockIdx.z;
+    int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int g = lane >> 4, col = lane & 15;
+    int group = hq / hkv;
+    int len = token_pos[t] + 1;
+    int lo = window > 0 ? max(0, len - window) : 0;
+    const int* pages = block_table + (size_t)token_seq[t] * bt_width;
+    int first_page = lo / AM_PAGE;
+    int n_pages = (len + AM_PAGE - 1) / AM_PAGE - first_page;
+    int per_split = (n_pages + n_splits - 1) / n_splits;
+    int p_begin = first_page + split * per_split;
+    int p_end = min(first_page + n_pages, p_begin + per_split);
+    int n_pieces = max(0, p_end - p_begin) * 2;
+
+    // Q^T operand: column = head of the group (zero beyond it), 8 values of D per lane and step.
+    bf16x8_t qf[KD];
+    {
+        bool ok = col < group;
+        const bf16_t* qrow = q + ((size_t)t * hq + kvh * group + (ok ? col : 0)) * D + g * 8;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) {
+            uint4 v = *(const uint4*)(qrow + kd * 32);
+            v.x = ok ? v.x : 0u; v.y = ok ? v.y : 0u; v.z = ok ? v.z : 0u; v.w = ok ? v.w : 0u;
+            qf[kd] = __builtin_bit_cast(bf16x8_t, v);
+        }
+    }
+    float m = -INFINITY, l = 0.f;
+    f32x4_t o[DT];
+#pragma unroll
+    for (int i = 0; i < DT; ++i) o[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    for (int piece = wave; piece < n_pieces; piece += 4) {
+        int lpage = p_begin + (piece >> 1), half = piece & 1;
+        int phys = pages[lpage];
+        const bf16_t* kbase = kcache + (((size_t)phys * hkv + kvh) * AM_PAGE + half * 32) * D;
+        const bf16_t* vbase = vcache + ((size_t)phys * hkv + kvh) * D * AM_PAGE + half * 32;
+        int key0 = lpage * AM_PAGE + half * 32;
+        // scores of 2 x 16 keys: element i of s[u] is key 16u + 4g + i, column = head.
+        f32x4_t s[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            s[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            const bf16_t* krow = kbase + (size_t)(u * 16 + col) * D + g * 8;
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) {
+                bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(krow + kd * 32));
+                s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[kd], s[u], 0, 0, 0);
+            }
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                int key = key0 + u * 16 + g * 4 + i;
+                float v = (key >= lo && key < len) ? s[u][i] * scale_log2e : -INFINITY;
+                s[u][i] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        float m_new = fmaxf(m, mx);
+        float m_use = m_new == -INFINITY ? 0.f : m_new;
+        float corr = fast_exp2(m - m_use);
+        float sum = 0.f;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                s[u][i] = fast_exp2(s[u][i] - m_use);
+                sum += s[u][i];
+            }
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        l = l * corr + sum;
+        m = m_new;
+        // P^T operand: slots 0..3 = keys 4g..4g+3, slots 4..7 = keys 16+4g..16+4g+3.
+        uint4 pv = make_uint4(pack_bf16x2(s[0][0], s[0][1]), pack_bf16x2(s[0][2], s[0][3]),
+                              pack_bf16x2(s[1][0], s[1][1]), pack_bf16x2(s[1][2], s[1][3]));
+        bf16x8_t pf = __builtin_bit_cast(bf16x8_t, pv);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const bf16_t* vrow = vbase + (size_t)(dt * 16 + col) * AM_PAGE + g * 4;
+            uint2 a = *(const uint2*)vrow, b = *(const uint2*)(vrow + 16);
+            bf16x8_t vf = __builtin_bit_cast(bf16x8_t, make_uint4(a.x, a.y, b.x, b.y));
+            o[dt] = o[dt] * corr;
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[dt], 0, 0, 0);
+        }
+    }
+    // merge the four waves in wave order; element i of o[dt] is d = 16 dt + 4g + i, column = head.
+    if (col < group) {
+        float* mine = sm_o + ((size_t)wave * group + col) * (D + 4);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) mine[dt * 16 + g * 4 + i] = o[dt][i];
+    }
+    if (g == 0) {
+        sm_m[wave][col] = m;
+        sm_l[wave][col] = l;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < group * D; idx += AM_THREADS) {
+        int head = idx / D, d = idx - head * D;
+        float mm = fmaxf(fmaxf(sm_m[0][head], sm_m[1][head]), fmaxf(sm_m[2][head], sm_m[3][head]));
+        float ll = 0.f, acc = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            float wgt = sm_m[w][head] == -INFINITY ? 0.f : fast_exp2(sm_m[w][head] - mm);
+            ll += sm_l[w][head] * wgt;
+            acc += sm_o[((size_t)w * group + head) * (D + 4) + d] * wgt;
+        }
+        int h = kvh * group + head;
+        if (n_splits == 1) {
+            out[((size_t)t * hq + h) * D + d] = f32_to_bf16(acc / ll);
+        } else {
+            size_t slot = ((size_t)t * hq + h) * n_splits + split;
+            part_o[slot * D + d] = acc;
+            if (d == 0) {
+                part_ml[slot * 2] = mm;
+                part_ml[slot * 2 + 1] = ll;
+            }
+        }
+    }
+}
+
+// Log-sum-exp merge of the splits in split order (rocml-kernels/kernels/attn_decode.hip:219-255).
+template <int D>
+__global__ void attn_decode_reduce_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                          bf16_t* __restrict__ out, int n_splits) {
+    int row = blockIdx.x;     // token * Hq + head
+    const float* ml = part_ml + (size_t)row * n_splits * 2;
+    float mm = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, ml[s * 2]);
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        float ll = 0.f, acc = 0.f;
+        for (int s = 0; s < n_splits; ++s) {
+            float wgt = ml[s * 2] == -INFINITY ? 0.f : fast_exp2(ml[s * 2] - mm);
+            ll += ml[s * 2 + 1] * wgt;
+            acc += part_o[((size_t)row * n_splits + s) * D + d] * wgt;
+        }
+        out[(size_t)row * D + d] = f32_to_bf16(acc / ll);
+    }
+}
+
+// ---- prefill: many query tokens per sequence --------------------------------------------------
+// grid (query tiles of 128 rows over all sequences, Hq), 4 waves of 32 query rows.  Pages of
+// keys and values go through LDS once per block; every wave multiplies its 32 queries with them.
+template <int D>
+struct PrefillLds {
+    static constexpr int K_ROW = D + 8;                 // bf16 per key row (16 bytes of padding)
+    static constexpr int V_ROW = AM_PAGE + 4;           // bf16 per value row (8 bytes of padding)
+    static constexpr int BYTES = (AM_PAGE * K_ROW + D * V_ROW) * 2;
+};
+
+template <int D>
+__global__ void __launch_bounds__(AM_THREADS)
+attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
+                         const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
+                         const int* __restrict__ block_table, int bt_width,
+                         const int* __restrict__ cu_seqlens, int n_seqs,
+                         const int* __restrict__ token_pos, int hq, int hkv, float scale_log2e,
+                         int window) {
+    using L = PrefillLds<D>;
+    constexpr int KK = D / 16;      // MFMA steps along D for the scores
+    constexpr int DT = D / 32;      // 32-row tiles of the output
+    extern __shared__ uint4 am_smem[];
+    bf16_t* sk = (bf16_t*)am_smem;
+    bf16_t* sv = sk + AM_PAGE * L::K_ROW;
+    int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int h2 = lane >> 5, col = lane & 31;
+    int h = blockIdx.y, kvh = h / (hq / hkv);
+    // which sequence and which of its query tiles
+    int tile = blockIdx.x, b = 0, tok0 = 0, n_new = 0;
+    for (; b < n_seqs; ++b) {
+        tok0 = cu_seqlens[b];
+        n_new = cu_seqlens[b + 1] - tok0;
+        int tiles = (n_new + 127) / 128;
+        if (tile < tiles) break;
+        tile -= tiles;
+    }
+    if (b >= n_seqs) return;
+    const int* pages = block_table + (size_t)b * bt_width;
+    int pos0 = token_pos[tok0];                        // position of the sequence's first new token
+    int row_lo = tile * 128, row_hi = min(n_new, row_lo + 128) - 1;     // block's query rows
+    int w_lo = row_lo + wave * 32, w_hi = min(n_new - 1, w_lo + 31);    // wave's query rows
+    bool wave_active = w_lo < n_new;
+    int my_row = w_lo + col;
+    bool row_ok = my_row < n_new;
+    int my_pos = pos0 + my_row;
+    int my_lo = window > 0 ? max(0, my_pos - window + 1) : 0;
+    int blk_first_key = window > 0 ? max(0, pos0 + row_lo - window + 1) : 0;
+    int blk_last_key = pos0 + row_hi;
+    int wave_first_key = window > 0 ? max(0, pos0 + w_lo - window + 1) : 0;
+    int wave_last_key = pos0 + w_hi;
+
+    // Q^T operand: column = query row, 8 values of D per lane and step.
+    bf16x8_t qf[KK];
+    {
+        const bf16_t* qrow = q + ((size_t)(tok0 + (row_ok ? my_row : 0)) * hq + h) * D + h2 * 8;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            uint4 v = *(const uint4*)(qrow + kk * 16);
+            v.x = row_ok ? v.x : 0u; v.y = row_ok ? v.y : 0u; v.z = row_ok ? v.z : 0u; v.w = row_ok ? v.w : 0u;
+            qf[kk] = __builtin_bit_cast(bf16x8_t, v);
+        }
+    }
+    float m = -INFINITY, l = 0.f;
+    f32x16_t o[DT];
+#pragma unroll
+    for (int i = 0; i < DT; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[i][e] = 0.f;
+
+    for (int lpage = blk_first_key / AM_PAGE; lpage <= blk_last_key / AM_PAGE; ++lpage) {
+        int phys = pages[lpage];
+        const uint4* gk = (const uint4*)(kcache + ((size_t)phys * hkv + kvh) * AM_PAGE * D);
+        const uint4* gv = (const uint4*)(vcache + ((size_t)phys * hkv + kvh) * D * AM_PAGE);
+        __syncthreads();                                // the previous page has been consumed
+        constexpr int K_PIECES = AM_PAGE * D / 8, V_PIECES = D * AM_PAGE / 8;
+#pragma unroll
+        for (int i = 0; i < K_PIECES / AM_THREADS; ++i) {
+            int piece = tid + i * AM_THREADS;
+            int key = piece / (D / 8), dc = piece % (D / 8);
+            *(uint4*)(sk + key * L::K_ROW + dc * 8) = gk[piece];
+        }
+#pragma unroll
+        for (int i = 0; i < V_PIECES / AM_THREADS; ++i) {
+            int piece = tid + i * AM_THREADS;
+            int d = piece / 8, kc = piece % 8;
+            uint4 v = gv[piece];
+            uint2* dst = (uint2*)(sv + d * L::V_ROW + kc * 8);
+            dst[0] = make_uint2(v.x, v.y);
+            dst[1] = make_uint2(v.z, v.w);
+        }
+        __syncthreads();
+        if (!wave_active) continue;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            int key0 = lpage * AM_PAGE + half * 32;
+            if (key0 > wave_last_key || key0 + 31 < wave_first_key) continue;   // wave-uniform
+            // S^T: element e of s is key 8(e/4) + 4 h2 + e%4, column = query row.
+            f32x16_t s;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s[e] = 0.f;
+            const bf16_t* krow = sk + (half * 32 + col) * L::K_ROW + h2 * 8;
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) {
+                bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(krow + kk * 16));
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], s, 0, 0, 0);
+            }
+            float mx = -INFINITY;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                int key = key0 + 8 * (e >> 2) + 4 * h2 + (e & 3);
+                float v = (row_ok && key <= my_pos && key >= my_lo) ? s[e] * scale_log2e : -INFINITY;
+                s[e] = v;
+                mx = fmaxf(mx, v);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            float m_new = fmaxf(m, mx);
+            float m_use = m_new == -INFINITY ? 0.f : m_new;
+            float corr = fast_exp2(m - m_use);
+            float sum = 0.f;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                s[e] = fast_exp2(s[e] - m_use);
+                sum += s[e];
+            }
+            sum += __shfl_xor(sum, 32, 64);
+            l = l * corr + sum;
+            m = m_new;
+            // P^T operands: MFMA u takes elements 8u..8u+7 = keys 16u + {4 h2 .. +3, 8 + 4 h2 .. +3}.
+            bf16x8_t pf[2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+                pf[u] = __builtin_bit_cast(bf16x8_t, make_uint4(
+                    pack_bf16x2(s[8 * u + 0], s[8 * u + 1]), pack_bf16x2(s[8 * u + 2], s[8 * u + 3]),
+                    pack_bf16x2(s[8 * u + 4], s[8 * u + 5]), pack_bf16x2(s[8 * u + 6], s[8 * u + 7])));
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) o[dt][e] *= corr;
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const bf16_t* vrow = sv + (dt * 32 + col) * L::V_ROW + half * 32 + 16 * u + 4 * h2;
+                    uint2 a = *(const uint2*)vrow, c = *(const uint2*)(vrow + 8);
+                    bf16x8_t vf = __builtin_bit_cast(bf16x8_t, make_uint4(a.x, a.y, c.x, c.y));
+                    o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[u], o[dt], 0, 0, 0);
+                }
+            }
+        }
+    }
+    if (!row_ok) return;
+    float inv = 1.0f / l;
+    bf16_t* orow = out + ((size_t)(tok0 + my_row) * hq + h) * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int e4 = 0; e4 < 4; ++e4) {
+            int d = dt * 32 + 8 * e4 + 4 * h2;
+            uint2 v = make_uint2(pack_bf16x2(o[dt][4 * e4] * inv, o[dt][4 * e4 + 1] * inv),
+                                 pack_bf16x2(o[dt][4 * e4 + 2] * inv, o[dt][4 * e4 + 3] * inv));
+            *(uint2*)(orow + d) = v;
+        }
+}

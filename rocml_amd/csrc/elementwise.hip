@@ -157,7 +157,8 @@ ROCML_EXPORT int rocml_rope_table(const int* pos, const double* inv_freq, float*
 // (rocml/src/forward/attention.rs:105-123), rotated with NEOX pairing (i, i + rot/2)
 // (rocml-kernels/kernels/rope.hip:18-33); q goes to q_out, k and v go straight into the
 // paged cache at the token's position (rocml-kernels/kernels/chunk_reshape.hip:37-74 is the
-// reference's separate scatter).  Cache layout: [page, Hkv, page_size, D].
+// reference's separate scatter).  Cache layout: keys [page, Hkv, page_size, D], values
+// transposed inside a page [page, Hkv, D, page_size] (what the MFMA attention kernels read).
 constexpr int QK_MAX_PER_LANE = 8;   // D <= 512
 constexpr int QK_WAVES = EW_BLOCK / WAVE;
 
@@ -229,8 +230,17 @@ __global__ void qk_norm_rope_append_kernel(
         int pos = token_pos[t];
         int page = block_table[(size_t)token_seq[t] * bt_width + pos / page_size];
         if (page < 0) return;
-        TO* base = kind == 1 ? kcache : vcache;
-        dst = base + (((size_t)page * hkv + head) * page_size + pos % page_size) * d;
+        if (kind == 2) {
+            // values are stored transposed inside a page: [page, Hkv, D, page_size]
+            TO* vdst = vcache + ((size_t)page * hkv + head) * d * page_size + pos % page_size;
+#pragma unroll
+            for (int j = 0; j < QK_MAX_PER_LANE; ++j) {
+                int e = lane + j * WAVE;
+                if (e < d) Elem<TO>::store(vdst + (size_t)e * page_size, v[j]);
+            }
+            return;
+        }
+        dst = kcache + (((size_t)page * hkv + head) * page_size + pos % page_size) * d;
     }
 #pragma unroll
     for (int j = 0; j < QK_MAX_PER_LANE; ++j) {

@@ -146,6 +146,7 @@ class Engine:
         step = StepContext(n_tokens=int(ids.size), n_seqs=len(slots), token_ids=d_ids, token_seq=d_seq,
                            token_pos=d_pos, cu_seqlens=d_cu, seq_lens=d_lens, seq_slots=d_slots,
                            max_new=max(len(t) for t in tokens), max_len=int(lens.max()),
+                           total_q_tiles=sum((len(t) + 127) // 128 for t in tokens),
                            workspace=self.workspace)
         return self.model.forward(step, self.cache, block_tables, d_want if want_rows.size else None,
                                   int(want_rows.size))

@@ -39,8 +39,8 @@ _SIGNATURES = {
         "rocml_gemm": [_P, _I, _I, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _LL, _P],
     },
     "attention": {
-        "rocml_attention": [_P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P,
-                            _LL, _P],
+        "rocml_attention": [_P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I,
+                            _P, _I, _I, _I, _I, _I, _P, _LL, _P],
     },
     "sampling": {
         "rocml_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P],
@@ -169,7 +169,8 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
                         v_cache: Optional[torch.Tensor], block_table: Optional[torch.Tensor],
                         token_seq: torch.Tensor, token_pos: torch.Tensor, write_kv: bool = True) -> None:
     """``qkv`` is ``[T, ld]`` with q, k, v side by side (k and v may be absent when
-    ``write_kv`` is false).  Caches are ``[pages, Hkv, page_size, D]``."""
+    ``write_kv`` is false).  Keys are ``[pages, Hkv, page_size, D]``, values
+    ``[pages, Hkv, D, page_size]``."""
     _dev(qkv, q_gain, k_gain, cos, sin, q_out, k_cache, v_cache, block_table, token_seq, token_pos)
     n_tokens, ld = qkv.shape
     for g in (q_gain, k_gain):
@@ -187,7 +188,8 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
     if write_kv:
         if k_cache is None or v_cache is None or block_table is None:
             raise KernelError("appending to the cache needs the cache and the block table")
-        if k_cache.shape[1:] != (n_kv_heads, k_cache.shape[2], head_dim) or v_cache.shape != k_cache.shape:
+        if k_cache.shape[1:] != (n_kv_heads, k_cache.shape[2], head_dim) \
+                or v_cache.shape != (k_cache.shape[0], n_kv_heads, head_dim, k_cache.shape[2]):
             raise KernelError(f"cache shape {tuple(k_cache.shape)} does not fit {n_kv_heads} heads of {head_dim}")
         if k_cache.dtype != q_out.dtype:
             raise KernelError("cache and q output must share their type")
@@ -233,30 +235,43 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
 
 
 # ---- attention -----------------------------------------------------------------------
-ATTN_AUTO, ATTN_PLAIN = 0, 1
+ATTN_AUTO, ATTN_PLAIN, ATTN_MFMA = 0, 1, 2
 
 
 def attention(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
               block_table: torch.Tensor, token_seq: torch.Tensor, token_pos: torch.Tensor,
               n_heads: int, n_kv_heads: int, head_dim: int, scale: float, window: Optional[int] = None,
-              algo: int = ATTN_AUTO, workspace: Optional[torch.Tensor] = None) -> None:
-    _dev(q, out, k_cache, v_cache, block_table, token_seq, token_pos)
+              algo: int = ATTN_AUTO, workspace: Optional[torch.Tensor] = None,
+              cu_seqlens: Optional[torch.Tensor] = None, max_new: int = 0, total_q_tiles: int = 0,
+              max_len: int = 0, n_splits: int = 0) -> None:
+    """Attention of the step's query tokens over the cache.  Keys are ``[pages, Hkv, page, D]``,
+    values ``[pages, Hkv, D, page]``.  ``cu_seqlens``, ``max_new`` (most query tokens of a
+    sequence), ``total_q_tiles`` (sum of ceil(tokens / 128)) and ``max_len`` (longest context)
+    describe the step to the fast kernels; without them the plain kernel runs."""
+    _dev(q, out, k_cache, v_cache, block_table, token_seq, token_pos, cu_seqlens)
     n_tokens = q.shape[0]
     if q.shape != (n_tokens, n_heads * head_dim) or out.shape != q.shape or out.dtype != q.dtype:
         raise KernelError("attention input and output must both be [tokens, heads * head_dim] of one type")
-    if k_cache.dtype != q.dtype or v_cache.shape != k_cache.shape \
-            or k_cache.shape[1] != n_kv_heads or k_cache.shape[3] != head_dim:
-        raise KernelError(f"cache {tuple(k_cache.shape)} {k_cache.dtype} does not fit the queries")
+    page = k_cache.shape[2]
+    if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype \
+            or k_cache.shape[1:] != (n_kv_heads, page, head_dim) \
+            or v_cache.shape != (k_cache.shape[0], n_kv_heads, head_dim, page):
+        raise KernelError(f"cache {tuple(k_cache.shape)} / {tuple(v_cache.shape)} {k_cache.dtype} does not fit the queries")
     _want(block_table, torch.int32, "block table")
     _want(token_seq, torch.int32, "token sequence table")
     _want(token_pos, torch.int32, "token position table")
     if token_seq.numel() != n_tokens or token_pos.numel() != n_tokens:
         raise KernelError("one sequence index and one position per token are needed")
+    n_seqs = 0
+    if cu_seqlens is not None:
+        _want(cu_seqlens, torch.int32, "sequence offsets")
+        n_seqs = cu_seqlens.numel() - 1
     ws_ptr, ws_bytes = (None, 0) if workspace is None else (workspace.data_ptr(), workspace.numel() * workspace.element_size())
     _check("attention", library("attention").rocml_attention(
         _ptr(q), _ptr(out), _ptr(k_cache), _ptr(v_cache), _code(q), _ptr(block_table),
         block_table.shape[1], _ptr(token_seq), _ptr(token_pos), n_tokens, n_heads, n_kv_heads, head_dim,
-        k_cache.shape[2], scale, 0 if window is None else int(window), algo, ws_ptr, ws_bytes, _stream()))
+        page, scale, 0 if window is None else int(window), algo, _ptr(cu_seqlens), n_seqs, max_new,
+        total_q_tiles, max_len, n_splits, ws_ptr, ws_bytes, _stream()))
 
 
 # ---- sampling ------------------------------------------------------------------------

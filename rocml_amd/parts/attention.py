@@ -82,7 +82,9 @@ class Attention(Mixer):
                                 step.token_pos, write_kv=owns_cache)
         o = ws.get("attn.o", (n, self.q_dim), self.dtype)
         ops.attention(q, o, cache.k, cache.v, cache.block_table, step.token_seq, step.token_pos,
-                      s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, workspace=ws.scratch())
+                      s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, workspace=ws.scratch(),
+                      cu_seqlens=step.cu_seqlens, max_new=step.max_new, total_q_tiles=step.total_q_tiles,
+                      max_len=step.max_len)
         ops.gemm(o, self.w_o, x_accum, accumulate=True, workspace=ws.scratch())
 
 

@@ -1,0 +1,173 @@
+"""The attention kernels alone against plain softmax attention written here, at other
+sizes than the engine's.  Shapes follow the reference's kernel tests
+(rocml-kernels/tests/attn_decode.rs:198-256, attn_prefill.rs:153-202): one cached
+position, lengths that are no multiple of a tile, several splits with a remainder, group
+sizes 1, 2 and 4, a head size of 256, a cache much longer than the sequence, a chunk that
+starts deep in the sequence.  Pages of the cache are handed out in a scrambled order and
+unused pages hold large values, so a read outside a sequence's pages or beyond its
+length shows.
+"""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from rocml_amd import ops  # noqa: E402
+
+PAGE = 64
+PLAIN, MFMA = 1, 2
+
+
+def _reference(q, k, v, positions, scale, window):
+    """q [n, Hq, D] for the tokens at ``positions`` of one sequence; k, v [L, Hkv, D]."""
+    n, hq, d = q.shape
+    group = hq // k.shape[1]
+    out = torch.zeros(n, hq, d, dtype=torch.float64)
+    for i, p in enumerate(positions):
+        lo = 0 if window is None else max(0, p - window + 1)
+        for h in range(hq):
+            s = (k[lo:p + 1, h // group].double() @ q[i, h].double()) * scale
+            w = torch.softmax(s, dim=0)
+            out[i, h] = w @ v[lo:p + 1, h // group].double()
+    return out
+
+
+def _build(seqs, hq, hkv, d, dtype, seed, spare_pages=3):
+    """seqs: list of (context length after the step, new tokens).  Returns device tensors of a
+    packed step and the per-sequence K, V, Q on the CPU."""
+    g = torch.Generator().manual_seed(seed)
+    n_pages = sum((length + PAGE - 1) // PAGE for length, _ in seqs) + spare_pages
+    order = torch.randperm(n_pages, generator=g).tolist()
+    kc = torch.full((n_pages, hkv, PAGE, d), 1e4, dtype=dtype)
+    vc = torch.full((n_pages, hkv, d, PAGE), 1e4, dtype=dtype)
+    width = max((length + PAGE - 1) // PAGE for length, _ in seqs)
+    table = torch.full((len(seqs), width), -1, dtype=torch.int32)
+    ks, vs, qs, tok_seq, tok_pos, cu = [], [], [], [], [], [0]
+    for b, (length, n_new) in enumerate(seqs):
+        k = torch.randn(length, hkv, d, generator=g).to(dtype)
+        v = torch.randn(length, hkv, d, generator=g).to(dtype)
+        q = torch.randn(n_new, hq, d, generator=g).to(dtype)
+        for lp in range((length + PAGE - 1) // PAGE):
+            page = order.pop()
+            table[b, lp] = page
+            rows = slice(lp * PAGE, min(length, (lp + 1) * PAGE))
+            n = rows.stop - rows.start
+            kc[page, :, :n] = k[rows].transpose(0, 1)
+            vc[page, :, :, :n] = v[rows].permute(1, 2, 0)
+            # the rest of the sequence's last page stays finite, as in the engine's cache
+            kc[page, :, n:] = 0
+            vc[page, :, :, n:] = 0
+        ks.append(k), vs.append(v), qs.append(q)
+        tok_seq += [b] * n_new
+        tok_pos += list(range(length - n_new, length))
+        cu.append(cu[-1] + n_new)
+    dev = dict(q=torch.cat(qs).reshape(-1, hq * d).cuda(), kc=kc.cuda(), vc=vc.cuda(), table=table.cuda(),
+               tok_seq=torch.tensor(tok_seq, dtype=torch.int32).cuda(),
+               tok_pos=torch.tensor(tok_pos, dtype=torch.int32).cuda(),
+               cu=torch.tensor(cu, dtype=torch.int32).cuda())
+    return dev, ks, vs, qs
+
+
+def _run(dev, seqs, hq, hkv, d, scale, window, algo, n_splits=0):
+    out = torch.full_like(dev["q"], float("nan"))
+    ws = torch.empty(32 << 20, dtype=torch.uint8, device="cuda")
+    ops.attention(dev["q"], out, dev["kc"], dev["vc"], dev["table"], dev["tok_seq"], dev["tok_pos"], hq, hkv,
+                  d, scale, window, algo=algo, workspace=ws, cu_seqlens=dev["cu"],
+                  max_new=max(n for _, n in seqs), total_q_tiles=sum((n + 127) // 128 for _, n in seqs),
+                  max_len=max(length for length, _ in seqs), n_splits=n_splits)
+    return out.cpu()
+
+
+def _check(seqs, hq, hkv, d, dtype, algo, window=None, n_splits=0, seed=0):
+    dev, ks, vs, qs = _build(seqs, hq, hkv, d, dtype, seed)
+    scale = 1.0 / math.sqrt(d)
+    got = _run(dev, seqs, hq, hkv, d, scale, window, algo, n_splits).double().reshape(-1, hq, d)
+    at = 0
+    tol = 1e-4 if dtype == torch.float32 else 1.5e-2     # bfloat16: probabilities and output are rounded
+    for (length, n_new), k, v, q in zip(seqs, ks, vs, qs):
+        ref = _reference(q, k, v, list(range(length - n_new, length)), scale, window)
+        err = float((got[at:at + n_new] - ref).abs().max())
+        assert err < tol, f"sequence of {length} with {n_new} new tokens: error {err}"
+        at += n_new
+
+
+# (Hq, Hkv, D, context length, splits): rocml-kernels/tests/attn_decode.rs:198-256
+DECODE = [(16, 8, 128, 1, 0), (16, 8, 128, 3, 0), (16, 8, 128, 33, 0), (16, 8, 128, 257, 1), (16, 8, 128, 257, 4),
+          (16, 8, 128, 2048, 1), (16, 8, 128, 2048, 8), (8, 2, 256, 400, 0), (8, 2, 256, 1024, 6),
+          (8, 8, 128, 300, 0), (16, 8, 128, 100, 0), (6, 2, 32, 77, 3), (4, 1, 64, 130, 2), (16, 1, 64, 65, 0),
+          (12, 4, 96, 200, 0)]
+
+
+@pytest.mark.parametrize("hq,hkv,d,length,splits", DECODE)
+def test_decode_bfloat16_mfma(hq, hkv, d, length, splits):
+    _check([(length, 1)], hq, hkv, d, torch.bfloat16, MFMA, n_splits=splits)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hq,hkv,d,length,splits", DECODE[:4] + [(5, 5, 48, 70, 0), (4, 2, 16, 129, 0)])
+def test_decode_plain(hq, hkv, d, length, splits, dtype):
+    _check([(length, 1)], hq, hkv, d, dtype, PLAIN)
+
+
+def test_decode_batch_of_unequal_lengths_and_windows():
+    seqs = [(1, 1), (64, 1), (65, 1), (700, 1), (129, 1), (2, 1), (1000, 1)]
+    for window in (None, 1, 70, 128):
+        _check(seqs, 8, 2, 128, torch.bfloat16, MFMA, window=window, seed=3)
+        _check(seqs, 8, 2, 128, torch.bfloat16, MFMA, window=window, n_splits=5, seed=3)
+        _check(seqs[:5], 6, 3, 48, torch.float32, PLAIN, window=window, seed=4)
+
+
+# (Hq, Hkv, D, new tokens, first position): rocml-kernels/tests/attn_prefill.rs:153-202
+PREFILL = [(16, 8, 128, 1, 0), (16, 8, 128, 1, 99), (16, 8, 128, 17, 0), (8, 2, 256, 64, 0), (8, 2, 256, 64, 200),
+           (16, 4, 128, 33, 50), (8, 8, 128, 40, 0), (16, 8, 128, 256, 1024), (16, 4, 128, 13, 0),
+           (6, 2, 32, 130, 0), (4, 1, 64, 300, 77), (12, 4, 96, 129, 3)]
+
+
+@pytest.mark.parametrize("hq,hkv,d,n_new,first", PREFILL)
+def test_prefill_bfloat16_mfma(hq, hkv, d, n_new, first):
+    _check([(first + n_new, n_new)], hq, hkv, d, torch.bfloat16, MFMA)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hq,hkv,d,n_new,first", PREFILL[:3] + [(5, 5, 48, 70, 10), (4, 2, 16, 129, 0)])
+def test_prefill_plain(hq, hkv, d, n_new, first, dtype):
+    _check([(first + n_new, n_new)], hq, hkv, d, dtype, PLAIN)
+
+
+def test_prefill_batch_of_unequal_lengths_and_windows():
+    seqs = [(5, 5), (200, 130), (64, 64), (129, 1), (400, 257), (1, 1)]
+    for window in (None, 1, 24, 70, 200):
+        _check(seqs, 8, 2, 64, torch.bfloat16, MFMA, window=window, seed=5)
+        _check(seqs[:4], 6, 2, 48, torch.float32, PLAIN, window=window, seed=6)
+
+
+def test_a_far_key_decides():
+    """One key far back among hundreds carries almost all weight: scale the query and that
+    key so that its score stands out; the output must be that key's value row."""
+    hq, hkv, d, length = 8, 2, 128, 900
+    for algo, n_new in ((MFMA, 1), (MFMA, 40), (PLAIN, 1)):
+        dev, ks, vs, qs = _build([(length, n_new)], hq, hkv, d, torch.bfloat16, 7)
+        far = 37
+        q = torch.zeros(n_new, hq, d)
+        q[:, :, 5] = 40.0
+        k_row = torch.zeros(hkv, d)
+        k_row[:, 5] = 40.0
+        page = int(dev["table"][0, far // PAGE])
+        dev["q"] = q.reshape(n_new, hq * d).to(torch.bfloat16).cuda()
+        dev["kc"][page, :, far % PAGE] = k_row.to(torch.bfloat16).cuda()
+        got = _run(dev, [(length, n_new)], hq, hkv, d, 1.0, None, algo).double().reshape(n_new, hq, d)
+        want = vs[0][far].double()            # [Hkv, D]
+        for h in range(hq):
+            assert float((got[:, h] - want[h // (hq // hkv)]).abs().max()) < 2e-2
+
+
+def test_refusals():
+    from rocml_amd.errors import KernelError
+    dev, *_ = _build([(10, 1)], 4, 2, 48, torch.bfloat16, 0)
+    with pytest.raises(KernelError):
+        _run(dev, [(10, 1)], 4, 2, 48, 1.0, None, MFMA)      # head size 48 has no MFMA kernel
+    dev, *_ = _build([(10, 1)], 4, 3, 32, torch.bfloat16, 0)
+    with pytest.raises(KernelError):
+        _run(dev, [(10, 1)], 4, 3, 32, 1.0, None, PLAIN)     # 4 heads over 3 kv heads
