@@ -34,6 +34,9 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--prefill-runs", type=int, default=3)
+    ap.add_argument("--skip-prompts", action="store_true",
+                    help="profiling aid: give the sequences their 2,048 positions without running the "
+                         "prompts (the cache holds zeros); the timed decode steps are the same")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this library")
@@ -73,8 +76,9 @@ def main() -> int:
         sync()
         engine.release(slot)
 
-    prefill_once()
-    times = []
+    if args.prefill_runs > 0:
+        prefill_once()
+    times = [float("nan")] if args.prefill_runs <= 0 else []
     for _ in range(args.prefill_runs):
         sync()
         t0 = time.perf_counter()
@@ -97,11 +101,16 @@ def main() -> int:
         slots = [engine.new_sequence() for _ in range(batch)]
         greedy = [SequenceSampling.start(SamplingParams.greedy(), i, []) for i in range(batch)]
         # Prompts go in a few at a time: the prefill is not what is timed here.
-        logits_rows = []
-        for i in range(0, batch, 4):
-            part = slots[i:i + 4]
-            logits_rows.append(engine.step([StepEntry(s, prompt(), [PROMPT_LEN - 1]) for s in part]).clone())
-        tokens = sampler.sample(torch.cat(logits_rows), greedy)
+        if args.skip_prompts:
+            engine.cache.reserve(slots, [PROMPT_LEN] * batch)
+            engine.cache.commit(slots, [PROMPT_LEN] * batch)
+            tokens = [1] * batch
+        else:
+            logits_rows = []
+            for i in range(0, batch, 4):
+                part = slots[i:i + 4]
+                logits_rows.append(engine.step([StepEntry(s, prompt(), [PROMPT_LEN - 1]) for s in part]).clone())
+            tokens = sampler.sample(torch.cat(logits_rows), greedy)
 
         def one_step(toks):
             logits = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, toks)])

@@ -172,18 +172,34 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
 template <int D>
 __global__ void attn_decode_reduce_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                           bf16_t* __restrict__ out, int n_splits) {
+    // At most 64 splits: lane s of every wave fetches split s's maximum and sum, so the loads
+    // go out together; the weights then sit in LDS for the sum over splits.
+    __shared__ float wgt[64];
     int row = blockIdx.x;     // token * Hq + head
     const float* ml = part_ml + (size_t)row * n_splits * 2;
-    float mm = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, ml[s * 2]);
+    int lane = threadIdx.x & 63;
+    bool has = lane < n_splits;
+    float ms = has ? ml[lane * 2] : -INFINITY;
+    float ls = has ? ml[lane * 2 + 1] : 0.f;
+    float mm = wave_max(ms);
+    float w = ms == -INFINITY ? 0.f : fast_exp2(ms - mm);
+    if (threadIdx.x < 64) wgt[lane] = w;
+    float inv_l = 1.0f / wave_sum(ls * w);          // every wave computes the same sum
+    __syncthreads();
+    const float* po = part_o + (size_t)row * n_splits * D;
     for (int d = threadIdx.x; d < D; d += blockDim.x) {
-        float ll = 0.f, acc = 0.f;
-        for (int s = 0; s < n_splits; ++s) {
-            float wgt = ml[s * 2] == -INFINITY ? 0.f : fast_exp2(ml[s * 2] - mm);
-            ll += ml[s * 2 + 1] * wgt;
-            acc += part_o[((size_t)row * n_splits + s) * D + d] * wgt;
+        float acc = 0.f;
+        int s = 0;
+        for (; s + 4 <= n_splits; s += 4) {
+            float a0 = po[(size_t)s * D + d], a1 = po[(size_t)(s + 1) * D + d];
+            float a2 = po[(size_t)(s + 2) * D + d], a3 = po[(size_t)(s + 3) * D + d];
+            acc += a0 * wgt[s];
+            acc += a1 * wgt[s + 1];
+            acc += a2 * wgt[s + 2];
+            acc += a3 * wgt[s + 3];
         }
-        out[(size_t)row * D + d] = f32_to_bf16(acc / ll);
+        for (; s < n_splits; ++s) acc += po[(size_t)s * D + d] * wgt[s];
+        out[(size_t)row * D + d] = f32_to_bf16(acc * inv_l);
     }
 }
 

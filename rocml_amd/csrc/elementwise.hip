@@ -75,12 +75,68 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restr
     for (int i = threadIdx.x; i < n; i += EW_BLOCK) Elem<TO>::store(o + i, xin[i] * inv * gain[i]);
 }
 
+// Same result for rows of up to 8192 values that are a multiple of 4: the row stays in
+// registers between the two passes and all loads are issued at once (a loop of single loads
+// waits for each one in turn, which is what a one-row decode step would spend its time on).
+constexpr int RN_VEC = 8;
+
+__device__ __forceinline__ void store4(float* p, float a, float b, float c, float d) {
+    *(float4*)p = make_float4(a, b, c, d);
+}
+__device__ __forceinline__ void store4(bf16_t* p, float a, float b, float c, float d) {
+    uint2 v;
+    v.x = (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+    v.y = (uint32_t)f32_to_bf16(c) | ((uint32_t)f32_to_bf16(d) << 16);
+    *(uint2*)p = v;
+}
+
+template <typename TO>
+__global__ void __launch_bounds__(EW_BLOCK)
+rmsnorm_vec_kernel(const float* __restrict__ x, const float* __restrict__ gain, TO* __restrict__ out,
+                   const int* __restrict__ rows, int n, float eps) {
+    __shared__ float scratch[EW_BLOCK / WAVE];
+    int r = blockIdx.x;
+    int src = rows ? rows[r] : r;
+    const float4* xin = (const float4*)(x + (size_t)src * n);
+    const float4* g4 = (const float4*)gain;
+    TO* o = out + (size_t)r * n;
+    int nv = n / 4;
+    float4 v[RN_VEC], g[RN_VEC];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < RN_VEC; ++j) {
+        int idx = threadIdx.x + j * EW_BLOCK;
+        bool ok = idx < nv;
+        v[j] = xin[ok ? idx : 0];
+        g[j] = g4[ok ? idx : 0];
+        if (!ok) v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int j = 0; j < RN_VEC; ++j)
+        ss = fmaf(v[j].x, v[j].x, fmaf(v[j].y, v[j].y, fmaf(v[j].z, v[j].z, fmaf(v[j].w, v[j].w, ss))));
+    float total = block_sum(ss, scratch);
+    float inv = 1.0f / sqrtf(total / (float)n + eps);
+#pragma unroll
+    for (int j = 0; j < RN_VEC; ++j) {
+        int idx = threadIdx.x + j * EW_BLOCK;
+        if (idx < nv)
+            store4(o + 4 * idx, v[j].x * inv * g[j].x, v[j].y * inv * g[j].y, v[j].z * inv * g[j].z,
+                   v[j].w * inv * g[j].w);
+    }
+}
+
 ROCML_EXPORT int rocml_rmsnorm(const float* x, const float* gain, void* out, int out_dtype,
                                const int* rows, int n_rows, int n, float eps, hipStream_t stream) {
     ROCML_REQUIRE(n_rows >= 0 && n > 0, "rmsnorm: bad sizes rows=%d n=%d", n_rows, n);
     ROCML_REQUIRE(eps > 0.f, "rmsnorm: eps must be positive, got %g", (double)eps);
     if (n_rows == 0) return 0;
-    if (out_dtype == ROCML_F32)
+    bool vec = n % 4 == 0 && n <= 4 * RN_VEC * EW_BLOCK && (uintptr_t)x % 16 == 0 &&
+               (uintptr_t)gain % 16 == 0 && (uintptr_t)out % 16 == 0;
+    if (vec && out_dtype == ROCML_F32)
+        rmsnorm_vec_kernel<float><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (float*)out, rows, n, eps);
+    else if (vec && out_dtype == ROCML_BF16)
+        rmsnorm_vec_kernel<bf16_t><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (bf16_t*)out, rows, n, eps);
+    else if (out_dtype == ROCML_F32)
         rmsnorm_kernel<float><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (float*)out, rows, n, eps);
     else if (out_dtype == ROCML_BF16)
         rmsnorm_kernel<bf16_t><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (bf16_t*)out, rows, n, eps);

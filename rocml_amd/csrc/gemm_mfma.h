@@ -250,6 +250,16 @@ __global__ void gemm_splitk_reduce_kernel(const float* __restrict__ partial, voi
     if (idx >= (long long)m * n) return;
     int gm = (int)(idx / n), gn = (int)(idx - (long long)gm * n);
     float s = 0.f;
-    for (int i = 0; i < splits; ++i) s += partial[(size_t)i * m * n + idx];
+    size_t stride = (size_t)m * n;
+    int i = 0;
+    for (; i + 4 <= splits; i += 4) {      // four loads in flight, added in split order
+        float a0 = partial[i * stride + idx], a1 = partial[(i + 1) * stride + idx];
+        float a2 = partial[(i + 2) * stride + idx], a3 = partial[(i + 3) * stride + idx];
+        s += a0;
+        s += a1;
+        s += a2;
+        s += a3;
+    }
+    for (; i < splits; ++i) s += partial[i * stride + idx];
     epilogue_store<EPI>(out, (size_t)gm * ldo + gn, s);
 }

@@ -40,6 +40,8 @@ class StepContext:
     total_q_tiles: int           # sum over sequences of ceil(new tokens / 128)
     workspace: Workspace
     memo: Dict = field(default_factory=dict)
+    block_tables: Dict = field(default_factory=dict)   # cache group name -> [B, width] int32
+    want_rows: Optional[torch.Tensor] = None           # token rows whose logits are wanted
 
     @property
     def is_decode(self) -> bool:

@@ -33,7 +33,7 @@ def _bucket(n: int) -> int:
 
 class Engine:
     def __init__(self, model: DecoderModel, max_tokens: int, max_seqs: Optional[int] = None,
-                 max_step_tokens: int = 8192):
+                 max_step_tokens: int = 8192, use_graphs: bool = True):
         if model.embed is None:
             raise RocmlError("the model has no weights bound")
         self.model = model
@@ -41,6 +41,9 @@ class Engine:
         self.workspace = Workspace(model.device)
         self.max_step_tokens = max_step_tokens
         self.steps_run = 0
+        self.use_graphs = use_graphs
+        self.max_graph_batch = 256
+        self._graphs: Dict[tuple, tuple] = {}
 
     # -- sequences -----------------------------------------------------------------------
     def new_sequence(self) -> int:
@@ -135,18 +138,54 @@ class Engine:
         host = np.concatenate(parts) if parts else np.zeros(0, np.int32)
         meta = self.workspace.get("step.meta", (max(host.size, 1),), torch.int32)
         meta[:host.size].copy_(torch.from_numpy(host))
-        views, at = [], 0
-        for p in parts:
-            views.append(meta[at:at + p.size])
-            at += p.size
-        d_ids, d_seq, d_pos, d_cu, d_lens, d_slots, d_want = views[:7]
-        block_tables: Dict[str, torch.Tensor] = {}
-        for g, v in zip(self.cache.kv_groups, views[7:]):
-            block_tables[g.name] = v.view(len(slots), width)
-        step = StepContext(n_tokens=int(ids.size), n_seqs=len(slots), token_ids=d_ids, token_seq=d_seq,
-                           token_pos=d_pos, cu_seqlens=d_cu, seq_lens=d_lens, seq_slots=d_slots,
-                           max_new=max(len(t) for t in tokens), max_len=int(lens.max()),
-                           total_q_tiles=sum((len(t) + 127) // 128 for t in tokens),
-                           workspace=self.workspace)
-        return self.model.forward(step, self.cache, block_tables, d_want if want_rows.size else None,
-                                  int(want_rows.size))
+        max_new = max(len(t) for t in tokens)
+        n_want = int(want_rows.size)
+
+        def context() -> StepContext:
+            views, at = [], 0
+            for p in parts:
+                views.append(meta[at:at + p.size])
+                at += p.size
+            d_ids, d_seq, d_pos, d_cu, d_lens, d_slots, d_want = views[:7]
+            block_tables: Dict[str, torch.Tensor] = {}
+            for g, v in zip(self.cache.kv_groups, views[7:]):
+                block_tables[g.name] = v.view(len(slots), width)
+            step = StepContext(n_tokens=int(ids.size), n_seqs=len(slots), token_ids=d_ids, token_seq=d_seq,
+                               token_pos=d_pos, cu_seqlens=d_cu, seq_lens=d_lens, seq_slots=d_slots,
+                               max_new=max_new, max_len=int(lens.max()),
+                               total_q_tiles=sum((len(t) + 127) // 128 for t in tokens),
+                               workspace=self.workspace)
+            step.block_tables = block_tables
+            step.want_rows = d_want if n_want else None
+            return step
+
+        def run(step: StepContext) -> Optional[torch.Tensor]:
+            return self.model.forward(step, self.cache, step.block_tables, step.want_rows, n_want)
+
+        if not (self.use_graphs and max_new == 1 and len(slots) <= self.max_graph_batch):
+            return run(context())
+        # Decode steps of one shape run from a recorded graph: the launches of a step are the
+        # same every time, only the integer tables change, and those lie at fixed addresses.
+        # A shape runs plainly the first time (kernels set themselves up, buffers reach their
+        # size), is recorded the second time, and replayed from then on.
+        key = (len(slots), n_want, width)
+        entry = self._graphs.get(key)
+        if entry is not None and entry[0] != self.workspace.generation:
+            entry = None                      # a buffer moved: the recorded addresses are stale
+        if entry is None:
+            result = run(context())
+            self._graphs[key] = (self.workspace.generation, None, None)
+            return result
+        generation, graph, result = entry
+        if graph is None:
+            graph = torch.cuda.CUDAGraph()
+            step = context()
+            with torch.cuda.graph(graph):
+                result = run(step)
+            if self.workspace.generation != generation:
+                # recording allocated a buffer after all; run plainly and start over
+                del self._graphs[key]
+                return run(context())
+            self._graphs[key] = (generation, graph, result)
+        graph.replay()
+        return result

@@ -63,6 +63,15 @@ class Attention(Mixer):
     def cache_request(self) -> KVCacheRequest:
         return KVCacheRequest(self.spec.n_kv_heads, self.spec.head_dim, self.spec.window)
 
+    def _decode_splits(self, step, cache) -> int:
+        """Splits of the key range in a decode step: enough blocks to fill the chip, at most one
+        per page the block table has room for.  It depends on the step's shape only, never on
+        the sequences' lengths, so a recorded step can be replayed as they grow."""
+        if step.max_new != 1:
+            return 0
+        blocks = step.n_tokens * self.spec.n_kv_heads
+        return max(1, min(512 // blocks, cache.block_table.shape[1], 64))
+
     def forward(self, step, xn, x_accum, cache, owns_cache: bool) -> None:
         s = self.spec
         n = step.n_tokens
@@ -84,7 +93,7 @@ class Attention(Mixer):
         ops.attention(q, o, cache.k, cache.v, cache.block_table, step.token_seq, step.token_pos,
                       s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, workspace=ws.scratch(),
                       cu_seqlens=step.cu_seqlens, max_new=step.max_new, total_q_tiles=step.total_q_tiles,
-                      max_len=step.max_len)
+                      max_len=step.max_len, n_splits=self._decode_splits(step, cache))
         ops.gemm(o, self.w_o, x_accum, accumulate=True, workspace=ws.scratch())
 
 
