@@ -1,0 +1,106 @@
+"""The Python entry point: load a model, step it, generate with it.
+
+It follows the reference's library surface (rocml/src/lib.rs:25-38): ``resolve`` a name or
+a path, ``Model.load(path, options)``, the forward calls, ``reset`` and the ``generate``
+family, with ``SamplingParams`` and ``Rng`` beside them.  Differences come from batching:
+the forward call is ``step`` over several sequences, and ``generate`` takes a list of
+prompts (token ids) and returns one result per prompt.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Iterable, List, Optional, Sequence, Union
+
+from .config.catalog import DEFAULT_CTX, ModelEntry, Resolved, resolve
+from .engine import Engine, EngineBackend, GenerateStats, Generator, Request, Result, StepEntry
+from .errors import RocmlError
+from .sampling import SamplingParams
+
+
+@dataclass(frozen=True)
+class LoadOptions:
+    """Knobs fixed when a model is loaded (rocml/src/load_opts.rs:61-165 has ``ctx`` and the
+    cache type; a quantized cache is not offered here).  ``ctx`` is the longest sequence the
+    cache is sized for, ``max_batch`` the most sequences that run together; the cache holds
+    ``ctx * max_batch`` positions unless ``max_tokens`` says otherwise."""
+    dtype: str = "bfloat16"
+    ctx: Optional[int] = None
+    max_batch: int = 8
+    max_tokens: Optional[int] = None
+    device: str = "cuda:0"
+    seed: int = 0                 # for models without a file (random weights)
+    use_graphs: bool = True
+
+
+class Model:
+    """A loaded model with its engine."""
+
+    def __init__(self, engine: Engine, options: LoadOptions, entry: Optional[ModelEntry]):
+        self.engine = engine
+        self.options = options
+        self.entry = entry
+        self.last_stats: Optional[GenerateStats] = None
+
+    @staticmethod
+    def load(name_or_path: str, options: Optional[LoadOptions] = None, **kwargs) -> "Model":
+        """``name_or_path`` is a folder with config.json and model.safetensors, or a catalog
+        name; a catalog model has no file and gets random weights from ``options.seed``."""
+        from .weights import load_model, random_model
+        options = options or LoadOptions(**kwargs)
+        found: Resolved = resolve(name_or_path)
+        if found.path is not None:
+            model = load_model(found.path, dtype=options.dtype, device=options.device)
+        else:
+            model = random_model(found.entry.config, seed=options.seed, dtype=options.dtype,
+                                 device=options.device, norm_jitter=found.entry.init_norm_jitter)
+        ctx = options.ctx or (found.entry.default_ctx if found.entry else DEFAULT_CTX)
+        ctx = min(ctx, model.spec.max_positions)
+        max_tokens = options.max_tokens or ctx * options.max_batch
+        engine = Engine(model, max_tokens=max_tokens, max_seqs=max(options.max_batch, 1),
+                        use_graphs=options.use_graphs)
+        return Model(engine, options, found.entry)
+
+    @property
+    def config(self):
+        return self.engine.model.config
+
+    @property
+    def vocab_size(self) -> int:
+        return self.engine.model.spec.vocab
+
+    def default_sampling(self) -> SamplingParams:
+        """The catalog's preset for this model, else greedy (flag > preset > greedy is the
+        command line's rule, rocml-cli/src/common.rs:167-176)."""
+        if self.entry is not None and self.entry.sampling is not None:
+            return self.entry.sampling
+        return SamplingParams.greedy()
+
+    # -- stepping ------------------------------------------------------------------------
+    def new_sequence(self) -> int:
+        return self.engine.new_sequence()
+
+    def release(self, slot: int) -> None:
+        self.engine.release(slot)
+
+    def step(self, entries: Sequence[StepEntry]):
+        return self.engine.step(entries)
+
+    # -- generation ----------------------------------------------------------------------
+    def generate(self, prompts: Sequence[Sequence[int]],
+                 sampling: Union[SamplingParams, Sequence[SamplingParams], None] = None,
+                 max_new_tokens: int = 64, stop_tokens: Iterable[int] = ()) -> List[Result]:
+        """Continues every prompt (lists of token ids).  ``sampling`` is one set of parameters
+        for all prompts or one per prompt; ``None`` means greedy.  A stop token ends its
+        sequence and is not part of the result."""
+        if sampling is None:
+            sampling = SamplingParams.greedy()
+        if isinstance(sampling, SamplingParams):
+            sampling = [sampling] * len(prompts)
+        if len(sampling) != len(prompts):
+            raise RocmlError("one SamplingParams for all prompts, or one per prompt")
+        stop = frozenset(int(t) for t in stop_tokens)
+        requests = [Request(list(p), max_new_tokens, s, stop) for p, s in zip(prompts, sampling)]
+        gen = Generator(EngineBackend(self.engine), max_batch=self.options.max_batch)
+        results = gen.run(requests)
+        self.last_stats = gen.stats
+        return results

@@ -1,0 +1,171 @@
+"""Command line in the manner of the reference's ``rocml-cli`` (rocml-cli/src/main.rs:25-48):
+the subcommands ``generate``, ``bench`` and ``models`` with its option names where it has
+them (rocml-cli/src/common.rs:38-57,146-177; cmd_generate.rs:19-49; cmd_bench.rs:15-77).
+Prompts are token ids (``--prompt-ids``); ``--prompt`` takes text when the model folder has a
+``tokenizer.json``.  There is no chat template, so ``--raw`` is accepted and changes nothing.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import statistics
+import sys
+import time
+from typing import List, Optional
+
+from ..errors import RocmlError
+
+
+def _add_model_args(p: argparse.ArgumentParser) -> None:
+    p.add_argument("--model", required=True, help="catalog name or a folder with config.json and model.safetensors")
+    p.add_argument("--no-download", action="store_true", help="accepted for compatibility; nothing is ever downloaded")
+    p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"],
+                   help="compute and cache type (the reference's --kv-cache picks its cache type)")
+    p.add_argument("--batch", type=int, default=8, help="most sequences that run together")
+
+
+def _add_sampling_args(p: argparse.ArgumentParser) -> None:
+    # Unset flags fall back to the model's catalog preset, then to greedy
+    # (rocml-cli/src/common.rs:167-176).
+    p.add_argument("-t", "--temperature", type=float, default=None)
+    p.add_argument("--top-p", type=float, default=None)
+    p.add_argument("--top-k", type=int, default=None)
+    p.add_argument("--seed", type=int, default=None)
+    p.add_argument("--repeat-penalty", type=float, default=None)
+
+
+def sampling_from_args(args, preset):
+    from ..sampling import SamplingParams
+    base = preset or SamplingParams()
+    return SamplingParams(
+        temperature=base.temperature if args.temperature is None else args.temperature,
+        top_k=base.top_k if args.top_k is None else args.top_k,
+        top_p=base.top_p if args.top_p is None else args.top_p,
+        seed=base.seed if args.seed is None else args.seed,
+        repeat_penalty=base.repeat_penalty if args.repeat_penalty is None else args.repeat_penalty,
+        repeat_penalty_window=base.repeat_penalty_window)
+
+
+def _parse_ids(text: str) -> List[int]:
+    return [int(t) for t in text.replace(",", " ").split()]
+
+
+def _load(args, ctx: Optional[int]):
+    from ..api import LoadOptions, Model
+    return Model.load(args.model, LoadOptions(dtype=args.dtype, ctx=ctx, max_batch=args.batch,
+                                              seed=getattr(args, "weights_seed", 0)))
+
+
+def _tokenizer(model_path: str):
+    import os
+    path = os.path.join(model_path, "tokenizer.json")
+    if not os.path.isfile(path):
+        raise RocmlError(f"--prompt needs {path}; give token ids with --prompt-ids instead")
+    from tokenizers import Tokenizer
+    return Tokenizer.from_file(path)
+
+
+def cmd_generate(args) -> int:
+    prompts: List[List[int]] = [_parse_ids(p) for p in (args.prompt_ids or [])]
+    tok = None
+    if args.prompt is not None:
+        tok = _tokenizer(args.model)
+        prompts.append(tok.encode(args.prompt).ids)
+    if not prompts:
+        raise RocmlError("give --prompt-ids (token ids) or --prompt (text, with a tokenizer.json)")
+    model = _load(args, args.ctx)
+    params = sampling_from_args(args, model.entry.sampling if model.entry else None)
+    results = model.generate(prompts, params, max_new_tokens=args.n, stop_tokens=_parse_ids(args.stop_ids or ""))
+    for i, r in enumerate(results):
+        if tok is not None and i == len(results) - 1 and args.prompt is not None:
+            print(tok.decode(r.tokens))
+        else:
+            print(" ".join(str(t) for t in r.tokens))
+    s = model.last_stats
+    print(f"prompt: {s.prompt_tokens} tokens in {s.prompt_seconds:.3f} s ({s.prompt_tok_s():.1f} tok/s); "
+          f"generated: {s.generated_tokens} tokens in {s.decode_seconds:.3f} s ({s.decode_tok_s():.1f} tok/s)",
+          file=sys.stderr)
+    return 0
+
+
+def cmd_bench(args) -> int:
+    """Synthetic prompt, greedy, no stop token, medians over runs
+    (rocml-cli/src/cmd_bench.rs:79-243)."""
+    import numpy as np
+    prompt_tokens = args.depth if args.depth is not None else args.prompt_tokens
+    ctx = args.ctx or max(4096, prompt_tokens + args.decode_tokens)
+    model = _load(args, ctx)
+    rng = np.random.default_rng(0)
+    prefill, decode = [], []
+    for _ in range(args.runs):
+        prompts = [[int(t) for t in rng.integers(0, model.vocab_size, size=prompt_tokens)]
+                   for _ in range(args.batch)]
+        model.generate(prompts, max_new_tokens=args.decode_tokens)
+        s = model.last_stats
+        prefill.append(s.prompt_tok_s())
+        decode.append(s.decode_tok_s())
+    out = {"model": args.model, "dtype": args.dtype, "batch": args.batch, "prompt_tokens": prompt_tokens,
+           "decode_tokens": args.decode_tokens, "runs": args.runs,
+           "prefill_tok_s": statistics.median(prefill), "decode_tok_s": statistics.median(decode)}
+    if args.json:
+        print(json.dumps(out))
+    else:
+        print(f"{args.model} {args.dtype} batch {args.batch}: prefill {out['prefill_tok_s']:.1f} tok/s "
+              f"({prompt_tokens} tokens), decode {out['decode_tok_s']:.1f} tok/s ({args.decode_tokens} tokens), "
+              f"median of {args.runs}")
+    return 0
+
+
+def cmd_models(args) -> int:
+    """Lists the catalog (rocml-cli/src/cmd_models.rs:13-38 prints name, family, presence)."""
+    from ..config import Qwen3Config
+    from ..config.catalog import CATALOG
+    print(f"{'name':<12} {'architecture':<18} {'layers':>6} {'hidden':>6} {'heads':>7} {'head':>5} "
+          f"{'inter':>6} {'vocab':>7} {'params':>9} {'bf16 GB':>8}")
+    for e in CATALOG:
+        c = Qwen3Config.from_dict(e.config)
+        print(f"{e.name:<12} {c.architectures[0]:<18} {c.num_hidden_layers:>6} {c.hidden_size:>6} "
+              f"{c.num_attention_heads:>3}/{c.num_key_value_heads:<3} {c.head_dim:>5} {c.intermediate_size:>6} "
+              f"{c.vocab_size:>7} {c.n_params() / 1e9:>8.3f}B {c.n_params() * 2 / 1e9:>8.2f}")
+    return 0
+
+
+def build_parser() -> argparse.ArgumentParser:
+    ap = argparse.ArgumentParser(prog="rocml_amd", description="Qwen3 generation on one MI355X")
+    sub = ap.add_subparsers(dest="command", required=True)
+    g = sub.add_parser("generate", help="continue prompts")
+    _add_model_args(g)
+    g.add_argument("--prompt", default=None, help="prompt text (needs tokenizer.json in the model folder)")
+    g.add_argument("--prompt-ids", action="append", help="prompt as token ids, e.g. '1 2 3'; repeat for a batch")
+    g.add_argument("--raw", action="store_true", help="accepted for compatibility: prompts are always raw")
+    g.add_argument("-n", "--max-tokens", dest="n", type=int, default=64)
+    g.add_argument("--ctx", type=int, default=None, help="longest sequence the cache is sized for")
+    g.add_argument("--stop-ids", default=None, help="token ids that end a sequence")
+    g.add_argument("--weights-seed", type=int, default=0, help="seed of the random weights of a catalog model")
+    _add_sampling_args(g)
+    g.set_defaults(fn=cmd_generate)
+    b = sub.add_parser("bench", help="measure prefill and decode speed")
+    _add_model_args(b)
+    b.add_argument("--prompt-tokens", type=int, default=64)
+    b.add_argument("--decode-tokens", type=int, default=128)
+    b.add_argument("--runs", type=int, default=3)
+    b.add_argument("--depth", type=int, default=None, help="prompt of this many tokens, then decode")
+    b.add_argument("--ctx", type=int, default=None)
+    b.add_argument("--json", action="store_true")
+    b.set_defaults(fn=cmd_bench)
+    m = sub.add_parser("models", help="list the catalog")
+    m.set_defaults(fn=cmd_models)
+    return ap
+
+
+def main(argv=None) -> int:
+    args = build_parser().parse_args(argv)
+    try:
+        return args.fn(args)
+    except RocmlError as e:
+        print(f"error: {e}", file=sys.stderr)
+        return 1
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -81,7 +81,7 @@ static int launch_skinny_m(const void* x, int ldx, const void* w, int ldw, void*
     return launch_skinny<4, EPI>(x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, stream);
 }
 
-// algo: 0 = choose, 1 = plain tiled kernel, 2 = MFMA tile kernel, 3 = MFMA few-rows kernel.
+// algo: 0 = choose, 1 = plain tiled kernel, 2 = MFMA tile kernel, 3 = MFMA few-rows kernel (M <= 64).
 // accumulate: out += product (out must be 32-bit); this is the residual sum's epilogue.
 // workspace: device memory for split-K partial sums (may be null: no split).
 ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, int w_dtype, int ldw,
@@ -97,7 +97,7 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
     bool bf16_in = x_dtype == ROCML_BF16 && w_dtype == ROCML_BF16;
     bool mfma_ok = bf16_in && k % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 &&
                    ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
-    if (algo == ALGO_MFMA_TILE || algo == ALGO_MFMA_SKINNY)
+    if (algo >= ALGO_MFMA_TILE)
         ROCML_REQUIRE(mfma_ok, "gemm: the MFMA kernels need bfloat16 operands, K and row strides that are "
                                "multiples of 8 and 16-byte aligned pointers (K=%d ldx=%d ldw=%d)", k, ldx, ldw);
     if (algo == ALGO_MFMA_SKINNY)

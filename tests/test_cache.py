@@ -1,0 +1,129 @@
+"""The cache's bookkeeping (no GPU): no slot or page is lost, held twice or freed twice;
+groups have storage of their own; a window gives pages back early; state starts at zero."""
+import random
+
+import pytest
+import torch
+
+from rocml_amd.cache import Cache, SlotAllocator, pages_for
+from rocml_amd.errors import CacheFullError, RocmlError
+from rocml_amd.parts import KVCacheRequest, StateRequest
+
+FULL = KVCacheRequest(2, 16, None)
+WIN = KVCacheRequest(2, 16, 100)
+STATE = StateRequest((3, 4))
+
+
+def _cache(requests, max_tokens, **kw):
+    return Cache(requests, max_tokens, torch.float32, "cpu", **kw)
+
+
+def test_slot_allocator():
+    a = SlotAllocator(3)
+    s = [a.alloc(), a.alloc(), a.alloc()]
+    assert sorted(s) == [0, 1, 2]
+    with pytest.raises(CacheFullError):
+        a.alloc()
+    a.free(1)
+    with pytest.raises(RocmlError, match="freed twice"):
+        a.free(1)
+    assert a.alloc() == 1                      # a freed slot is used again at once
+    with pytest.raises(RocmlError):
+        a.free(7)
+
+
+def test_groups_have_their_own_storage_and_lines():
+    c = _cache([FULL, WIN, FULL, None, STATE, WIN], 64 * 10, max_seqs=4)
+    assert len(c.kv_groups) == 2 and len(c.state_groups) == 1
+    full, win = c.kv_groups
+    assert full.n_lines == 2 and win.n_lines == 2
+    assert full.k.shape == (2, 10, 2, 64, 16) and full.v.shape == (2, 10, 2, 16, 64)
+    assert win.n_pages == min(10, 4 * (pages_for(100) + 1))
+    assert c.line(0) == (full, 0) and c.line(2) == (full, 1) and c.line(5) == (win, 1)
+    assert not c.has_line(3)
+    assert c.state_groups[0].state.shape == (1, 4, 3, 4)
+    assert c.bytes_per_token() == 2 * (2 + 2) * 2 * 16 * 4
+
+
+def test_pages_follow_lengths_and_reserve_is_all_or_nothing():
+    c = _cache([FULL], 64 * 4)
+    a, b = c.new_sequence(), c.new_sequence()
+    c.reserve([a, b], [65, 64])
+    c.commit([a, b], [65, 64])
+    g = c.kv_groups[0]
+    assert len(g.page_table(a)) == 2 and len(g.page_table(b)) == 1 and g.n_free_pages == 1
+    with pytest.raises(CacheFullError):
+        c.reserve([a, b], [129, 129])          # needs 1 + 2 pages, 1 is free
+    assert g.n_free_pages == 1 and len(g.page_table(a)) == 2      # nothing was taken
+    c.reserve([a], [128])                      # no new page
+    assert g.n_free_pages == 1
+    c.check()
+    table = c.block_table(g, [b, a], 4)
+    assert table.shape == (2, 4) and list(table[0, 1:]) == [-1, -1, -1] and table[1, 1] >= 0
+    c.free_sequence(a)
+    with pytest.raises(RocmlError):
+        c.free_sequence(a)
+    assert g.n_free_pages == 3
+    c.check()
+
+
+def test_window_releases_pages_no_query_can_see():
+    c = _cache([WIN], 64 * 8)
+    s = c.new_sequence()
+    g = c.kv_groups[0]
+    c.reserve([s], [300])
+    assert g.n_free_pages == 8 - 5
+    c.commit([s], [300])
+    # a query at position 300 sees keys from 201 on: pages 0..2 (positions 0..191) are free again
+    assert g.page_table(s)[:3] == [-1, -1, -1] and g.page_table(s)[3] >= 0
+    assert g.n_free_pages == 6
+    c.reserve([s], [301])
+    c.commit([s], [301])
+    assert len(g.page_table(s)) == 5
+    c.check()
+    c.free_sequence(s)
+    assert g.n_free_pages == 8
+
+
+def test_state_is_zero_when_a_slot_is_handed_out():
+    c = _cache([STATE], 64 * 2, max_seqs=2)
+    s = c.new_sequence()
+    c.state_groups[0].state[:, s] = 5.0
+    c.free_sequence(s)
+    assert c.new_sequence() == s
+    assert float(c.state_groups[0].state[:, s].abs().max()) == 0.0
+
+
+def test_random_traffic_keeps_the_books_balanced():
+    rng = random.Random(0)
+    c = _cache([FULL, WIN], 64 * 40, max_seqs=12)
+    live = {}
+    for _ in range(3000):
+        op = rng.random()
+        if op < 0.25 and len(live) < 12:
+            live[c.new_sequence()] = 0
+        elif op < 0.4 and live:
+            s = rng.choice(list(live))
+            c.free_sequence(s)
+            del live[s]
+        elif live:
+            some = rng.sample(list(live), k=min(len(live), rng.randint(1, 4)))
+            new = [live[s] + rng.randint(1, 90) for s in some]
+            try:
+                c.reserve(some, new)
+            except CacheFullError:
+                c.check()
+                continue
+            c.commit(some, new)
+            for s, n in zip(some, new):
+                live[s] = n
+        c.check()
+        for s, n in live.items():
+            assert c.length(s) == n
+            for g in c.kv_groups:
+                table = g.page_table(s)
+                assert len(table) >= pages_for(n)
+                first = 0 if g.request.window is None else max(0, n - g.request.window + 1) // 64
+                assert all(p >= 0 for p in table[first:])          # every page a query may read is held
+    held = [p for g in c.kv_groups[:1] for s in live for p in g.page_table(s) if p >= 0]
+    assert len(held) == len(set(held))                              # no page held twice

@@ -1,0 +1,138 @@
+"""The generation loop's decisions with a scripted backend (no GPU): batches, stop tokens,
+sequences that end earlier, slots given back and used again, limits."""
+from typing import Dict, List
+
+import pytest
+
+from rocml_amd.engine.generate import Generator, Request
+from rocml_amd.errors import CacheFullError, RocmlError
+from rocml_amd.sampling import Rng, SamplingParams, sequence_seed
+
+
+class Scripted:
+    """Next token of a sequence = (sum of its tokens so far) % 50; counts what it is asked."""
+
+    def __init__(self, max_positions=1000, slots=4, room=10_000):
+        self.max_positions = max_positions
+        self.free_slots = list(range(slots))
+        self.room = room
+        self.history: Dict[int, List[int]] = {}
+        self.steps: List[List[int]] = []          # slots of each step
+        self.step_tokens: List[List[List[int]]] = []
+        self.released: List[int] = []
+
+    def can_admit(self, lengths):
+        return len(lengths) <= len(self.free_slots) and sum(lengths) <= self.room
+
+    def new_sequence(self):
+        s = self.free_slots.pop(0)
+        self.history[s] = []
+        return s
+
+    def release(self, slot):
+        assert slot in self.history, "released twice"
+        del self.history[slot]
+        self.released.append(slot)
+        self.free_slots.insert(0, slot)
+
+    def step(self, slots, tokens):
+        assert len(set(slots)) == len(slots)
+        self.steps.append(list(slots))
+        self.step_tokens.append([list(t) for t in tokens])
+        for s, t in zip(slots, tokens):
+            self.history[s].extend(t)
+        return [sum(self.history[s]) % 50 for s in slots]
+
+    def sample(self, logits, seqs):
+        return list(logits)
+
+    def synchronize(self):
+        pass
+
+
+def _expected(prompt, n, stop=()):
+    toks, out = list(prompt), []
+    for _ in range(n):
+        t = sum(toks) % 50
+        if t in stop:
+            return out, "stop"
+        out.append(t)
+        toks.append(t)
+    return out, "length"
+
+
+def test_unequal_prompts_end_at_different_times():
+    be = Scripted()
+    reqs = [Request([1, 2, 3], 5), Request([4], 2), Request([7, 7, 7, 7, 7, 7], 8), Request([9, 1], 1)]
+    res = Generator(be, max_batch=4).run(reqs)
+    for r, q in zip(res, reqs):
+        assert (r.tokens, r.finish_reason) == _expected(q.prompt, q.max_new_tokens)
+        assert r.prompt_tokens == len(q.prompt)
+    assert be.steps[0] == [0, 1, 2, 3] and be.step_tokens[0] == [[1, 2, 3], [4], [7] * 6, [9, 1]]
+    assert be.steps[1] == [0, 1, 2]              # the request with one new token has left
+    assert be.steps[2] == [0, 2]
+    assert all(len(t) == 1 for step in be.step_tokens[1:] for t in step)     # one token each afterwards
+    assert len(be.steps) == 8                    # prompt step + 7 more for the longest (no step after its last token)
+    assert sorted(be.released) == [0, 1, 2, 3] and not be.history
+
+
+def test_stop_token_is_not_emitted_and_frees_the_slot():
+    full, _ = _expected([5, 6], 10)
+    stop = full[3]
+    want, reason = _expected([5, 6], 10, stop=[stop])
+    be = Scripted()
+    res = Generator(be).run([Request([5, 6], 10, stop_tokens=frozenset([stop])), Request([1], 10)])
+    assert (res[0].tokens, res[0].finish_reason) == (want, "stop") and stop not in res[0].tokens
+    assert res[1].finish_reason == "length" and len(res[1].tokens) == 10
+    gone = len(want) + 1                          # steps in which the first sequence took part
+    assert all(0 in s for s in be.steps[:gone]) and all(0 not in s for s in be.steps[gone:])
+
+
+def test_batches_follow_slots_and_room_and_reuse_slots():
+    be = Scripted(slots=2)
+    reqs = [Request([i + 1], 3) for i in range(5)]
+    res = Generator(be, max_batch=8).run(reqs)
+    assert [r.tokens for r in res] == [_expected(q.prompt, 3)[0] for q in reqs]
+    assert sorted(be.steps[0]) == [0, 1] and sorted(be.steps[3]) == [0, 1] and len(be.steps[6]) == 1    # three batches
+    assert be.released.count(0) == 3 and be.released.count(1) == 2
+    be = Scripted(slots=8, room=20)               # room for prompt + output of two requests at a time
+    gen = Generator(be, max_batch=8)
+    gen.run([Request([1] * 4, 5)] * 5)
+    assert gen.stats.batches == 3
+    with pytest.raises(CacheFullError):
+        Generator(Scripted(room=5)).run([Request([1] * 4, 5)])
+    be = Scripted()
+    Generator(be, max_batch=1).run([Request([1], 1), Request([2], 1)])
+    assert [len(s) for s in be.steps] == [1, 1]
+
+
+def test_limits_and_empty_prompts():
+    be = Scripted(max_positions=6)
+    res = Generator(be).run([Request([1, 2, 3, 4], 10), Request([], 5), Request([3], 0)])
+    assert res[0].finish_reason == "context" and len(res[0].tokens) == 2      # 4 + 2 = 6 positions
+    assert res[1].finish_reason == "empty" and res[1].tokens == []
+    assert res[2].finish_reason == "length" and res[2].tokens == []
+    with pytest.raises(RocmlError, match="positions"):
+        Generator(be).run([Request([1] * 7, 1)])
+    with pytest.raises(RocmlError):
+        Generator(be, max_batch=0)
+
+
+def test_rng_matches_the_reference_generator():
+    # xorshift64* (rocml/src/sample.rs:56-83), first outputs for seed 1 computed by hand from
+    # the definition: x ^= x >> 12; x ^= x << 25; x ^= x >> 27; out = x * 0x2545F4914F6CDD1D.
+    r = Rng(1)
+    x = 1
+    x ^= x >> 12
+    x ^= (x << 25) & (2 ** 64 - 1)
+    x ^= x >> 27
+    assert r.next_u64() == (x * 0x2545F4914F6CDD1D) % 2 ** 64
+    assert Rng(0).state == 0x9E3779B97F4A7C15
+    draws = [Rng(42).next_f32() for _ in range(3)]
+    assert draws[0] == draws[1] == draws[2] and 0.0 <= draws[0] < 1.0
+    r = Rng(7)
+    vals = [r.next_f32() for _ in range(2000)]
+    assert 0.45 < sum(vals) / len(vals) < 0.55 and all(v * 2 ** 24 == int(v * 2 ** 24) for v in vals)
+    assert sequence_seed(5, 0) == 5 and len({sequence_seed(5, i) for i in range(100)}) == 100
+    assert SamplingParams().is_greedy() and not SamplingParams(temperature=0.7).is_greedy()
+    assert not SamplingParams(repeat_penalty=1.0).penalty_active() and SamplingParams(repeat_penalty=1.1).penalty_active()
