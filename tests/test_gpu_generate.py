@@ -1,0 +1,125 @@
+"""Generation through the Python entry point against the plain implementation: greedy
+tokens, stop tokens, more requests than fit one batch (slots are used again), long
+decoding, the first tokens of a sequence, seeded temperature sampling."""
+import pytest
+import torch
+
+from tests import helpers
+from tests.plain import qwen3_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    root = tmp_path_factory.mktemp("gen_models")
+    out = {}
+    for name, (cfg, seed) in helpers.TINY.items():
+        path = helpers.make_model_dir(root, cfg, seed, torch.float32)
+        out[name] = (path, helpers.read_config(path), helpers.read_weights(path))
+    return out
+
+
+def _load(path, dtype, **kw):
+    from rocml_amd.api import Model
+    return Model.load(path, dtype=dtype, **kw)
+
+
+def near_tie(cfg, weights, prompt, produced, k):
+    """The reference's rule for a greedy flip (rocml/tests/greedy_parity.rs:33-34,158-160):
+    acceptable only where the two best logits of the plain run are within 1e-2 of each
+    other, relative to the larger."""
+    logits = plain.forward(cfg, weights, list(prompt) + list(produced[:k]))[-1]
+    top = torch.topk(logits, 2).values
+    return float((top[0] - top[1]).abs() / top[0].abs().clamp_min(1e-9)) < 1e-2
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+def test_greedy_float32_matches_token_for_token(models, name):
+    path, cfg, weights = models[name]
+    model = _load(path, "float32", ctx=256, max_batch=3)
+    lengths = [5, 9, 13, 1, 30, 2, 64]
+    prompts = [helpers.random_tokens(n, cfg["vocab_size"], 40 + i) for i, n in enumerate(lengths)]
+    want = [plain.greedy(cfg, weights, p, 8) for p in prompts]
+    got = model.generate(prompts, max_new_tokens=8)            # 7 requests, 3 slots: three batches
+    assert [r.tokens for r in got] == want
+    assert all(r.finish_reason == "length" for r in got)
+    assert model.last_stats.batches == 3 and model.last_stats.generated_tokens == 56
+    model.engine.cache.check()
+    assert not model.engine.cache.lengths
+    # a stop token ends its sequence early and is not emitted; the others go on
+    stop = want[2][3]
+    got = model.generate(prompts[:3], max_new_tokens=8, stop_tokens=[stop])
+    for r, w, p in zip(got, want, prompts):
+        ref = plain.greedy(cfg, weights, p, 8, stop=[stop])
+        assert r.tokens == ref and r.finish_reason == ("stop" if len(ref) < 8 else "length")
+
+
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_greedy_bfloat16_flips_only_at_near_ties(models, name):
+    path, cfg, weights = models[name]
+    rounded = {k: (v if v.dim() == 1 else v.to(torch.bfloat16).float()) for k, v in weights.items()}
+    model = _load(path, "bfloat16", ctx=128, max_batch=4)
+    prompts = [helpers.random_tokens(n, cfg["vocab_size"], 60 + i) for i, n in enumerate([1, 7, 16, 33])]
+    got = [r.tokens for r in model.generate(prompts, max_new_tokens=12)]
+    for p, g in zip(prompts, got):
+        assert len(g) == 12
+        w = plain.greedy(cfg, rounded, p, 12)
+        if g != w:
+            k = next(i for i in range(12) if g[i] != w[i])
+            assert near_tie(cfg, rounded, p, w, k), f"tokens differ at {k} without a near tie: {g} vs {w}"
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 2e-2)])
+def test_long_decoding_and_first_tokens(models, dtype, tol):
+    from rocml_amd.engine import StepEntry
+    path, cfg, weights = models["D"]               # window of 70: decoding crosses pages and the window's edge
+    w = weights if dtype == "float32" else {k: (v if v.dim() == 1 else v.to(torch.bfloat16).float()) for k, v in weights.items()}
+    model = _load(path, dtype, ctx=512, max_batch=2)
+    toks = helpers.random_tokens(260, cfg["vocab_size"], 77)
+    ref = plain.forward(cfg, w, toks)
+    eng = model.engine
+    slot = eng.new_sequence()
+    rows = [eng.step([StepEntry(slot, toks[:3], [0, 1, 2])]).cpu()]
+    for t in toks[3:]:
+        rows.append(eng.step([StepEntry(slot, [t], [0])]).cpu())
+    eng.release(slot)
+    got = torch.cat(rows)
+    assert helpers.rel_to_max(got, ref) < tol
+    assert helpers.rel_to_max(got[:3], ref[:3]) < tol          # the first tokens of a sequence
+    # one token at a time from the very first token
+    slot = eng.new_sequence()
+    rows = [eng.step([StepEntry(slot, [t], [0])]).cpu() for t in toks[:5]]
+    eng.release(slot)
+    assert helpers.rel_to_max(torch.cat(rows), ref[:5]) < tol
+
+
+def test_temperature_sampling_is_seeded_and_ignores_batching(models):
+    from rocml_amd.sampling import SamplingParams
+    path, cfg, weights = models["B"]
+    prompts = [helpers.random_tokens(n, cfg["vocab_size"], 80 + i) for i, n in enumerate([1, 7, 16, 33])]
+    params = SamplingParams(temperature=0.7, seed=1)
+    together = _load(path, "float32", ctx=128, max_batch=4)
+    a = [r.tokens for r in together.generate(prompts, params, max_new_tokens=12)]
+    b = [r.tokens for r in together.generate(prompts, params, max_new_tokens=12)]
+    assert a == b
+    one_by_one = _load(path, "float32", ctx=128, max_batch=1)
+    c = [r.tokens for r in one_by_one.generate(prompts, params, max_new_tokens=12)]
+    assert a == c                                                # batches of one draw the same tokens
+    d = [r.tokens for r in together.generate(prompts, SamplingParams(temperature=0.7, seed=2), max_new_tokens=12)]
+    assert a != d
+    greedy = [r.tokens for r in together.generate(prompts, max_new_tokens=12)]
+    assert a != greedy
+
+
+def test_command_line_generate_and_models(models, capsys):
+    from rocml_amd.cli import main
+    path, cfg, weights = models["A"]
+    prompt = helpers.random_tokens(6, cfg["vocab_size"], 5)
+    rc = main(["generate", "--model", path, "--dtype", "float32", "--prompt-ids", " ".join(map(str, prompt)),
+               "-n", "5", "--ctx", "64", "--batch", "2"])
+    out = capsys.readouterr().out.strip().splitlines()
+    assert rc == 0 and [int(t) for t in out[-1].split()] == plain.greedy(cfg, weights, prompt, 5)
+    assert main(["models"]) == 0 and "qwen3-8b" in capsys.readouterr().out
+    assert main(["generate", "--model", "no-such-model", "--prompt-ids", "1"]) == 1
+    assert "known names" in capsys.readouterr().err
