@@ -1,0 +1,234 @@
+"""Each part alone against its plain formula, and what the layer list can express: a layer
+named twice, a layer that reads another layer's cache, and a toy mixer with state of its own
+that is defined here, registered, built and stepped without a change to the library."""
+import math
+from dataclasses import dataclass
+
+import pytest
+import torch
+
+from tests import helpers
+from tests.plain import qwen3_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+from rocml_amd.config.spec import (AttentionSpec, BlockSpec, GatedMlpSpec, ModelSpec, NormSpec, RopeSpec,  # noqa: E402
+                                   ScheduleEntry)
+
+
+def _tensors(model, seed, dtype_of=None):
+    from rocml_amd.weights.random_init import random_tensor
+    out = {}
+    for name, p in model.param_specs().items():
+        out[name] = random_tensor(name, p, seed, model.storage_dtype(p), True).to(model.device)
+    return out
+
+
+def _engine(spec, dtype, seed=0, **kw):
+    from rocml_amd.engine import DecoderModel, Engine
+    model = DecoderModel(spec, dtype, device="cuda:0")
+    tensors = _tensors(model, seed)
+    model.bind(tensors)
+    return Engine(model, max_tokens=2048, **kw), {k: v.cpu().double() for k, v in tensors.items()}
+
+
+def _spec(layers, schedule, hidden, vocab, tied=True):
+    return ModelSpec(architecture="test", vocab=vocab, hidden=hidden, layers=tuple(layers), schedule=tuple(schedule),
+                     final_norm=NormSpec(hidden, 1e-5), tie_lm_head=tied, max_positions=1024)
+
+
+def _attention_spec(hidden, hq, hkv, d, window=None, norm=True, theta=1e4, rot=None):
+    return AttentionSpec(hidden=hidden, n_heads=hq, n_kv_heads=hkv, head_dim=d, scale=1 / math.sqrt(d), window=window,
+                         qk_norm=NormSpec(d, 1e-5) if norm else None,
+                         position=RopeSpec(d, rot or d, theta) if theta else None)
+
+
+def _block(hidden, mixer, inter=48):
+    return BlockSpec(mixer=mixer, ffn=GatedMlpSpec(hidden, inter), mixer_norm=NormSpec(hidden, 1e-5),
+                     ffn_norm=NormSpec(hidden, 1e-5))
+
+
+# ---- plain versions of a block built from the parts' own parameter names --------------------
+def plain_attention(xn, w, pre, s, positions, k_cache=None):
+    t = xn.shape[0]
+    q = (xn @ w[pre + "q_proj.weight"].t()).reshape(t, s.n_heads, s.head_dim)
+    if k_cache is None:
+        k = (xn @ w[pre + "k_proj.weight"].t()).reshape(t, s.n_kv_heads, s.head_dim)
+        v = (xn @ w[pre + "v_proj.weight"].t()).reshape(t, s.n_kv_heads, s.head_dim)
+        if s.qk_norm is not None:
+            k = plain.rmsnorm(k, w[pre + "k_norm.weight"], s.qk_norm.eps)
+        if s.position is not None:
+            r = s.position.rot_dim
+            k = torch.cat([plain.rope_neox(k[..., :r], positions, s.position.theta), k[..., r:]], -1)
+    else:
+        k, v = k_cache
+    if s.qk_norm is not None:
+        q = plain.rmsnorm(q, w[pre + "q_norm.weight"], s.qk_norm.eps)
+    if s.position is not None:
+        r = s.position.rot_dim
+        q = torch.cat([plain.rope_neox(q[..., :r], positions, s.position.theta), q[..., r:]], -1)
+    o = plain.causal_attention(q, k, v, s.scale, s.window)
+    return o.reshape(t, -1) @ w[pre + "o_proj.weight"].t(), (k, v)
+
+
+def plain_model(spec, w, tokens):
+    x = w["embed.weight"][tokens]
+    positions = list(range(len(tokens)))
+    caches = {}
+    for i, e in enumerate(spec.schedule):
+        b = spec.layers[e.layer]
+        pre = f"layers.{e.layer}."
+        xn = plain.rmsnorm(x, w[pre + "mixer_norm.weight"], b.mixer_norm.eps)
+        out, kv = plain_attention(xn, w, pre + "mixer.", b.mixer, positions,
+                                  caches[e.reads_cache_of] if e.reads_cache_of is not None else None)
+        caches[i] = kv
+        x = x + out
+        xn = plain.rmsnorm(x, w[pre + "ffn_norm.weight"], b.ffn_norm.eps)
+        g = xn @ w[pre + "ffn.gate_proj.weight"].t()
+        u = xn @ w[pre + "ffn.up_proj.weight"].t()
+        x = x + plain.swiglu(g, u) @ w[pre + "ffn.down_proj.weight"].t()
+    xn = plain.rmsnorm(x, w["final_norm.weight"], spec.final_norm.eps)
+    return xn @ (w["embed.weight"] if spec.tie_lm_head else w["lm_head.weight"]).t()
+
+
+@pytest.mark.parametrize("mixer", [
+    _attention_spec(40, 5, 5, 16), _attention_spec(40, 4, 2, 32, window=9), _attention_spec(40, 6, 2, 48, norm=False),
+    _attention_spec(40, 2, 1, 64, theta=None), _attention_spec(40, 4, 4, 32, rot=16, theta=5e5),
+    _attention_spec(40, 8, 2, 128, window=70)])
+def test_attention_part_options(mixer):
+    """One block whose mixer has the option under test; whole and token by token."""
+    spec = _spec([_block(40, mixer)], [ScheduleEntry(0)], 40, 97)
+    for dtype, tol in (("float32", 2e-5), ("bfloat16", 2.5e-2)):
+        engine, w = _engine(spec, dtype, seed=3)
+        if dtype == "bfloat16":
+            w = {k: (v if v.dim() == 1 else v.float().to(torch.bfloat16).double()) for k, v in w.items()}
+        toks = helpers.random_tokens(90, 97, 1)
+        ref = plain_model(spec, w, toks)
+        assert helpers.rel_to_max(helpers.run_whole(engine, toks), ref) < tol
+        assert helpers.rel_to_max(helpers.run_tail_by_one(engine, toks, 32), ref) < tol
+
+
+def test_layer_named_twice_and_shared_cache():
+    a = _block(48, _attention_spec(48, 4, 2, 16))
+    b = _block(48, _attention_spec(48, 4, 2, 16, window=20), inter=80)
+    schedule = [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(1), ScheduleEntry(0, reads_cache_of=0)]
+    spec = _spec([a, b], schedule, 48, 131, tied=False)
+    engine, w = _engine(spec, "float32", seed=4)
+    assert len(engine.cache.kv_groups) == 2                          # full and windowed lines apart
+    assert engine.cache.kv_groups[0].n_lines == 1 and engine.cache.kv_groups[1].n_lines == 2
+    toks = helpers.random_tokens(70, 131, 2)
+    ref = plain_model(spec, w, toks)
+    assert helpers.rel_to_max(helpers.run_whole(engine, toks), ref) < 2e-5
+    assert helpers.rel_to_max(helpers.run_tail_by_one(engine, toks, 32), ref) < 2e-5
+    got = helpers.run_batch(engine, [toks, toks[:33], toks[:5]], [60, 20, 1])
+    for g, n in zip(got, (70, 33, 5)):
+        assert helpers.rel_to_max(g, ref[:n]) < 2e-5
+
+
+def test_norm_rope_and_mlp_parts_alone():
+    from rocml_amd.engine import Workspace
+    from rocml_amd.engine.batch import StepContext
+    from rocml_amd.parts import BuildContext, build_feed_forward, build_norm, build_position
+    ctx = BuildContext(dtype=torch.float32, device=torch.device("cuda:0"))
+    g = torch.Generator().manual_seed(0)
+    norm = build_norm(NormSpec(72, 3e-6), ctx)
+    gain = torch.randn(72, generator=g)
+    norm.bind({"weight": gain.cuda()})
+    x = torch.randn(9, 72, generator=g)
+    out = torch.empty(9, 72, device="cuda")
+    norm.forward(x.cuda(), out)
+    assert float((out.cpu().double() - plain.rmsnorm(x.double(), gain.double(), 3e-6)).abs().max()) < 1e-5
+    ffn = build_feed_forward(GatedMlpSpec(72, 100), ctx)
+    ws = {n: (torch.randn(p.shape, generator=g) * 0.1) for n, p in ffn.param_specs().items()}
+    ffn.bind({n: t.cuda() for n, t in ws.items()})
+    pos = torch.tensor([5, 6, 7, 0, 1, 2, 3, 4, 900], dtype=torch.int32).cuda()
+    step = StepContext(n_tokens=9, n_seqs=1, token_ids=pos, token_seq=pos, token_pos=pos, cu_seqlens=pos, seq_lens=pos,
+                       seq_slots=pos, max_new=9, max_len=9, total_q_tiles=1, workspace=Workspace("cuda:0"))
+    acc = x.cuda().clone()
+    ffn.forward(step, x.cuda(), acc)
+    xd = x.double()
+    want = xd + plain.swiglu(xd @ ws["gate_proj.weight"].double().t(), xd @ ws["up_proj.weight"].double().t()) \
+        @ ws["down_proj.weight"].double().t()
+    assert float((acc.cpu().double() - want).abs().max()) < 1e-5
+    rope = build_position(RopeSpec(32, 16, 7e4), ctx)
+    cos, sin = rope.tables(step)
+    assert rope.tables(step)[0] is cos                                  # one table per step, shared
+    ang = pos.cpu().double()[:, None] * torch.tensor([7e4 ** (-2.0 * i / 16) for i in range(8)], dtype=torch.float64)
+    assert float((cos.cpu().double() - ang.cos()).abs().max()) < 1e-7 and float((sin.cpu().double() - ang.sin()).abs().max()) < 1e-7
+
+
+# ---- a toy mixer with state of its own ---------------------------------------------------
+@dataclass(frozen=True)
+class DecaySpec:
+    hidden: int
+    width: int
+    decay: float
+    kind: str = "toy_decay"
+
+
+def _toy_parts():
+    from rocml_amd.parts import Mixer, ParamSpec, StateRequest, register_mixer
+
+    class DecayMixer(Mixer):
+        """state <- decay * state + W_in x, out = W_out state: a running sum per sequence,
+        kept in the cache's fixed-size state and advanced once per token, in order."""
+
+        def __init__(self, spec, ctx):
+            self.spec = spec
+
+        def param_specs(self):
+            s = self.spec
+            return {"in_proj.weight": ParamSpec((s.width, s.hidden)), "out_proj.weight": ParamSpec((s.hidden, s.width))}
+
+        def bind(self, tensors):
+            self.w_in, self.w_out = tensors["in_proj.weight"].float(), tensors["out_proj.weight"].float()
+
+        def cache_request(self):
+            return StateRequest((self.spec.width,))
+
+        def forward(self, step, xn, x_accum, cache, owns_cache):
+            u = xn.float() @ self.w_in.t()                      # [T, width]
+            slots = cache.slots.cpu().tolist()
+            cu = step.cu_seqlens.cpu().tolist()
+            for b, slot in enumerate(slots):
+                state = cache.state[slot]
+                for t in range(cu[b], cu[b + 1]):
+                    state.mul_(self.spec.decay).add_(u[t])
+                    x_accum[t] += state @ self.w_out.t()
+    register_mixer("toy_decay", DecayMixer)
+
+
+def test_toy_mixer_with_state_registers_builds_and_steps():
+    _toy_parts()
+    toy = _block(32, DecaySpec(32, 12, 0.9))
+    att = _block(32, _attention_spec(32, 2, 1, 16))
+    spec = _spec([toy, att, toy], [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2)], 32, 77)
+    engine, w = _engine(spec, "float32", seed=5, use_graphs=False)
+    assert len(engine.cache.state_groups) == 1 and engine.cache.state_groups[0].n_lines == 2
+
+    def reference(tokens):
+        x = w["embed.weight"][tokens]
+        for i, b in enumerate(spec.layers):
+            pre = f"layers.{i}."
+            xn = plain.rmsnorm(x, w[pre + "mixer_norm.weight"], 1e-5)
+            if b.mixer.kind == "toy_decay":
+                state = torch.zeros(12, dtype=torch.float64)
+                out = []
+                for t in range(len(tokens)):
+                    state = 0.9 * state + w[pre + "mixer.in_proj.weight"] @ xn[t]
+                    out.append(w[pre + "mixer.out_proj.weight"] @ state)
+                x = x + torch.stack(out)
+            else:
+                x = x + plain_attention(xn, w, pre + "mixer.", b.mixer, list(range(len(tokens))))[0]
+            xn = plain.rmsnorm(x, w[pre + "ffn_norm.weight"], 1e-5)
+            x = x + plain.swiglu(xn @ w[pre + "ffn.gate_proj.weight"].t(), xn @ w[pre + "ffn.up_proj.weight"].t()) \
+                @ w[pre + "ffn.down_proj.weight"].t()
+        return plain.rmsnorm(x, w["final_norm.weight"], 1e-5) @ w["embed.weight"].t()
+
+    a, b = helpers.random_tokens(40, 77, 6), helpers.random_tokens(23, 77, 7)
+    ra, rb = reference(a), reference(b)
+    assert helpers.rel_to_max(helpers.run_whole(engine, a), ra) < 1e-4
+    # the slot is handed out again: its state must start at zero
+    assert helpers.rel_to_max(helpers.run_tail_by_one(engine, b, 10), rb) < 1e-4
+    got = helpers.run_batch(engine, [a, b], [30, 3])
+    assert helpers.rel_to_max(got[0], ra) < 1e-4 and helpers.rel_to_max(got[1], rb) < 1e-4
