@@ -67,9 +67,18 @@ def library(family: str) -> ctypes.CDLL:
     return lib
 
 
-def load_all() -> None:
-    for family in _SIGNATURES:
+MODEL_FAMILIES = ("elementwise", "gemm", "attention")   # what a model's step needs; sampling comes with generation
+
+
+def prepare(families=tuple(_SIGNATURES)) -> None:
+    """Loads the named families; those that are not built yet are compiled together first."""
+    _build.build([f for f in families], force=False)
+    for family in families:
         library(family)
+
+
+def load_all() -> None:
+    prepare()
 
 
 def _check(family: str, status: int) -> None:
