@@ -57,22 +57,34 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 // ---- RMSNorm ---------------------------------------------------------------------
 // out[r, i] = x[src(r), i] * (1/sqrt(sum(x^2)/n + eps)) * gain[i]
 // (rocml-kernels/kernels/rmsnorm.hip:18-42).  `rows` optionally gathers source rows.
+// With `partials` ([n_splits][rows of x][n], the split-K partial sums of the product whose
+// result belongs to x) the kernel first forms x + sum of the partials in split order, which is
+// the residual sum the reference does in a kernel of its own
+// (rocml-kernels/kernels/elementwise.hip:7-12), writes it back to x unless rows are gathered,
+// and normalises that.
 template <typename TO>
-__global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ gain,
-                               TO* __restrict__ out, const int* __restrict__ rows, int n, float eps) {
+__global__ void rmsnorm_kernel(float* x, const float* __restrict__ gain, TO* __restrict__ out,
+                               const int* __restrict__ rows, int n, float eps,
+                               const float* __restrict__ partials, int n_splits, long long split_stride) {
     __shared__ float scratch[EW_BLOCK / WAVE];
     int r = blockIdx.x;
     int src = rows ? rows[r] : r;
-    const float* xin = x + (size_t)src * n;
+    float* xin = x + (size_t)src * n;
     TO* o = out + (size_t)r * n;
     float ss = 0.f;
     for (int i = threadIdx.x; i < n; i += EW_BLOCK) {
         float v = xin[i];
+        for (int sp = 0; sp < n_splits; ++sp) v += partials[sp * split_stride + (size_t)src * n + i];
+        if (n_splits > 0 && !rows) xin[i] = v;
         ss = fmaf(v, v, ss);
     }
     float total = block_sum(ss, scratch);
     float inv = 1.0f / sqrtf(total / (float)n + eps);
-    for (int i = threadIdx.x; i < n; i += EW_BLOCK) Elem<TO>::store(o + i, xin[i] * inv * gain[i]);
+    for (int i = threadIdx.x; i < n; i += EW_BLOCK) {
+        float v = xin[i];
+        if (rows) for (int sp = 0; sp < n_splits; ++sp) v += partials[sp * split_stride + (size_t)src * n + i];
+        Elem<TO>::store(o + i, v * inv * gain[i]);
+    }
 }
 
 // Same result for rows of up to 8192 values that are a multiple of 4: the row stays in
@@ -92,12 +104,13 @@ __device__ __forceinline__ void store4(bf16_t* p, float a, float b, float c, flo
 
 template <typename TO>
 __global__ void __launch_bounds__(EW_BLOCK)
-rmsnorm_vec_kernel(const float* __restrict__ x, const float* __restrict__ gain, TO* __restrict__ out,
-                   const int* __restrict__ rows, int n, float eps) {
+rmsnorm_vec_kernel(float* x, const float* __restrict__ gain, TO* __restrict__ out,
+                   const int* __restrict__ rows, int n, float eps, const float* __restrict__ partials,
+                   int n_splits, long long split_stride) {
     __shared__ float scratch[EW_BLOCK / WAVE];
     int r = blockIdx.x;
     int src = rows ? rows[r] : r;
-    const float4* xin = (const float4*)(x + (size_t)src * n);
+    float4* xin = (float4*)(x + (size_t)src * n);
     const float4* g4 = (const float4*)gain;
     TO* o = out + (size_t)r * n;
     int nv = n / 4;
@@ -110,6 +123,34 @@ rmsnorm_vec_kernel(const float* __restrict__ x, const float* __restrict__ gain, 
         v[j] = xin[ok ? idx : 0];
         g[j] = g4[ok ? idx : 0];
         if (!ok) v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    if (n_splits > 0) {
+        const float4* p4 = (const float4*)(partials + (size_t)src * n);
+        long long stride4 = split_stride / 4;
+        for (int sp = 0; sp < n_splits; sp += 2) {      // two splits' loads in flight, added in order
+            bool second = sp + 1 < n_splits;
+            float4 a[RN_VEC], c[RN_VEC];
+#pragma unroll
+            for (int j = 0; j < RN_VEC; ++j) {
+                int idx = threadIdx.x + j * EW_BLOCK;
+                int safe = idx < nv ? idx : 0;
+                a[j] = p4[sp * stride4 + safe];
+                c[j] = p4[(second ? sp + 1 : sp) * stride4 + safe];
+            }
+#pragma unroll
+            for (int j = 0; j < RN_VEC; ++j) {
+                if (threadIdx.x + j * EW_BLOCK >= nv) continue;
+                v[j].x += a[j].x; v[j].y += a[j].y; v[j].z += a[j].z; v[j].w += a[j].w;
+                if (second) { v[j].x += c[j].x; v[j].y += c[j].y; v[j].z += c[j].z; v[j].w += c[j].w; }
+            }
+        }
+        if (!rows) {
+#pragma unroll
+            for (int j = 0; j < RN_VEC; ++j) {
+                int idx = threadIdx.x + j * EW_BLOCK;
+                if (idx < nv) xin[idx] = v[j];
+            }
+        }
     }
 #pragma unroll
     for (int j = 0; j < RN_VEC; ++j)
@@ -125,23 +166,29 @@ rmsnorm_vec_kernel(const float* __restrict__ x, const float* __restrict__ gain, 
     }
 }
 
-ROCML_EXPORT int rocml_rmsnorm(const float* x, const float* gain, void* out, int out_dtype,
-                               const int* rows, int n_rows, int n, float eps, hipStream_t stream) {
+ROCML_EXPORT int rocml_rmsnorm(float* x, const float* gain, void* out, int out_dtype, const int* rows,
+                               int n_rows, int n, float eps, const float* partials, int n_splits,
+                               long long split_stride, hipStream_t stream) {
     ROCML_REQUIRE(n_rows >= 0 && n > 0, "rmsnorm: bad sizes rows=%d n=%d", n_rows, n);
     ROCML_REQUIRE(eps > 0.f, "rmsnorm: eps must be positive, got %g", (double)eps);
+    ROCML_REQUIRE(n_splits >= 0 && (n_splits == 0 || (partials && split_stride > 0)),
+                  "rmsnorm: partial sums need a pointer and a stride");
     if (n_rows == 0) return 0;
     bool vec = n % 4 == 0 && n <= 4 * RN_VEC * EW_BLOCK && (uintptr_t)x % 16 == 0 &&
-               (uintptr_t)gain % 16 == 0 && (uintptr_t)out % 16 == 0;
+               (uintptr_t)gain % 16 == 0 && (uintptr_t)out % 16 == 0 &&
+               (n_splits == 0 || ((uintptr_t)partials % 16 == 0 && split_stride % 4 == 0));
+#define RN_ARGS rows, n, eps, partials, n_splits, split_stride
     if (vec && out_dtype == ROCML_F32)
-        rmsnorm_vec_kernel<float><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (float*)out, rows, n, eps);
+        rmsnorm_vec_kernel<float><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (float*)out, RN_ARGS);
     else if (vec && out_dtype == ROCML_BF16)
-        rmsnorm_vec_kernel<bf16_t><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (bf16_t*)out, rows, n, eps);
+        rmsnorm_vec_kernel<bf16_t><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (bf16_t*)out, RN_ARGS);
     else if (out_dtype == ROCML_F32)
-        rmsnorm_kernel<float><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (float*)out, rows, n, eps);
+        rmsnorm_kernel<float><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (float*)out, RN_ARGS);
     else if (out_dtype == ROCML_BF16)
-        rmsnorm_kernel<bf16_t><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (bf16_t*)out, rows, n, eps);
+        rmsnorm_kernel<bf16_t><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (bf16_t*)out, RN_ARGS);
     else
         return rocml_fail("rmsnorm: unknown dtype code %d", out_dtype);
+#undef RN_ARGS
     ROCML_CHECK_LAUNCH("rmsnorm");
     return 0;
 }
@@ -149,31 +196,33 @@ ROCML_EXPORT int rocml_rmsnorm(const float* x, const float* gain, void* out, int
 // ---- gated activation ------------------------------------------------------------
 // out[t, i] = silu(gu[t, i]) * gu[t, inter + i],  silu(g) = g / (1 + exp(-g))
 // (rocml-kernels/kernels/silu_mul.hip:12-20).  Gate and up halves lie side by side in a row.
+// With `interleaved` a row holds (gate_0, up_0, gate_1, up_1, ...), the order the fused product
+// epilogue wants its weight rows in.
 template <typename TI, typename TO>
 __global__ void swiglu_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inter,
-                              long long total) {
+                              long long total, int interleaved) {
     long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
     if (idx >= total) return;
     long long t = idx / inter;
     int i = (int)(idx - t * inter);
     const TI* row = gu + (size_t)t * 2 * inter;
-    float g = Elem<TI>::load(row + i);
-    float u = Elem<TI>::load(row + inter + i);
+    float g = Elem<TI>::load(row + (interleaved ? 2 * i : i));
+    float u = Elem<TI>::load(row + (interleaved ? 2 * i + 1 : inter + i));
     Elem<TO>::store(out + idx, g / (1.0f + expf(-g)) * u);
 }
 
 ROCML_EXPORT int rocml_swiglu(const void* gu, int in_dtype, void* out, int out_dtype, int n_tokens,
-                              int inter, hipStream_t stream) {
+                              int inter, int interleaved, hipStream_t stream) {
     ROCML_REQUIRE(n_tokens >= 0 && inter > 0, "swiglu: bad sizes T=%d I=%d", n_tokens, inter);
     long long total = (long long)n_tokens * inter;
     if (total == 0) return 0;
     int grid = ceil_div(total, EW_BLOCK);
     if (in_dtype == ROCML_F32 && out_dtype == ROCML_F32)
-        swiglu_kernel<float, float><<<grid, EW_BLOCK, 0, stream>>>((const float*)gu, (float*)out, inter, total);
+        swiglu_kernel<float, float><<<grid, EW_BLOCK, 0, stream>>>((const float*)gu, (float*)out, inter, total, interleaved);
     else if (in_dtype == ROCML_F32 && out_dtype == ROCML_BF16)
-        swiglu_kernel<float, bf16_t><<<grid, EW_BLOCK, 0, stream>>>((const float*)gu, (bf16_t*)out, inter, total);
+        swiglu_kernel<float, bf16_t><<<grid, EW_BLOCK, 0, stream>>>((const float*)gu, (bf16_t*)out, inter, total, interleaved);
     else if (in_dtype == ROCML_BF16 && out_dtype == ROCML_BF16)
-        swiglu_kernel<bf16_t, bf16_t><<<grid, EW_BLOCK, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, total);
+        swiglu_kernel<bf16_t, bf16_t><<<grid, EW_BLOCK, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, total, interleaved);
     else
         return rocml_fail("swiglu: unsupported dtype pair in=%d out=%d", in_dtype, out_dtype);
     ROCML_CHECK_LAUNCH("swiglu");
@@ -211,7 +260,8 @@ ROCML_EXPORT int rocml_rope_table(const int* pos, const double* inv_freq, float*
 // One wave per (token, head row) of the packed projection output [T, (Hq + 2 Hkv) * D]:
 // q and k rows are normalised over D with one gain vector each
 // (rocml/src/forward/attention.rs:105-123), rotated with NEOX pairing (i, i + rot/2)
-// (rocml-kernels/kernels/rope.hip:18-33); q goes to q_out, k and v go straight into the
+// (rocml-kernels/kernels/rope.hip:18-33); with n_splits > 1 the input is the projection's split-K
+// partial sums [n_splits][T, ld], summed here in split order; q goes to q_out, k and v go straight into the
 // paged cache at the token's position (rocml-kernels/kernels/chunk_reshape.hip:37-74 is the
 // reference's separate scatter).  Cache layout: keys [page, Hkv, page_size, D], values
 // transposed inside a page [page, Hkv, D, page_size] (what the MFMA attention kernels read).
@@ -225,7 +275,7 @@ __global__ void qk_norm_rope_append_kernel(
     const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot,
     TO* __restrict__ q_out, TO* __restrict__ kcache, TO* __restrict__ vcache,
     const int* __restrict__ block_table, int bt_width, const int* __restrict__ token_seq,
-    const int* __restrict__ token_pos, int page_size, int write_kv) {
+    const int* __restrict__ token_pos, int page_size, int write_kv, int n_splits, long long split_stride) {
     extern __shared__ float stage[];   // [QK_WAVES][d]
     int wave = threadIdx.x / WAVE;
     int lane = threadIdx.x & (WAVE - 1);
@@ -242,7 +292,22 @@ __global__ void qk_norm_rope_append_kernel(
 #pragma unroll
     for (int j = 0; j < QK_MAX_PER_LANE; ++j) {
         int e = lane + j * WAVE;
-        v[j] = (active && e < d) ? Elem<TI>::load(src + e) : 0.f;
+        bool ok = active && e < d;
+        float val = Elem<TI>::load(ok ? src + e : qkv);
+        // split-K partial sums of the projection, added in split order
+        // (four loads in flight at a time)
+        for (int sp = 1; sp < n_splits; sp += 4) {
+            const TI* p = ok ? src + e : qkv;
+            float a0 = Elem<TI>::load(ok ? p + sp * split_stride : qkv);
+            float a1 = Elem<TI>::load(ok && sp + 1 < n_splits ? p + (sp + 1) * split_stride : qkv);
+            float a2 = Elem<TI>::load(ok && sp + 2 < n_splits ? p + (sp + 2) * split_stride : qkv);
+            float a3 = Elem<TI>::load(ok && sp + 3 < n_splits ? p + (sp + 3) * split_stride : qkv);
+            val += a0;
+            if (sp + 1 < n_splits) val += a1;
+            if (sp + 2 < n_splits) val += a2;
+            if (sp + 3 < n_splits) val += a3;
+        }
+        v[j] = ok ? val : 0.f;
         ss = fmaf(v[j], v[j], ss);
     }
     const float* gain = kind == 0 ? q_gain : (kind == 1 ? k_gain : nullptr);
@@ -309,8 +374,11 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     const void* qkv, int in_dtype, int ld, int n_tokens, int hq, int hkv, int d, const float* q_gain,
     const float* k_gain, float eps, const float* cos_t, const float* sin_t, int rot, void* q_out,
     void* kcache, void* vcache, int out_dtype, const int* block_table, int bt_width,
-    const int* token_seq, const int* token_pos, int page_size, int write_kv, hipStream_t stream) {
+    const int* token_seq, const int* token_pos, int page_size, int write_kv, int n_splits,
+    long long split_stride, hipStream_t stream) {
     ROCML_REQUIRE(n_tokens >= 0 && hq > 0 && hkv > 0 && d > 0, "qk_norm_rope_append: bad sizes");
+    ROCML_REQUIRE(n_splits >= 1 && (n_splits == 1 || (split_stride > 0 && in_dtype == ROCML_F32)),
+                  "qk_norm_rope_append: partial sums must be 32-bit with a positive stride");
     ROCML_REQUIRE(d <= QK_MAX_PER_LANE * WAVE, "qk_norm_rope_append: head_dim %d exceeds %d", d,
                   QK_MAX_PER_LANE * WAVE);
     ROCML_REQUIRE(ld >= (hq + 2 * hkv) * d || (!write_kv && ld >= hq * d),
@@ -326,7 +394,7 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     qk_norm_rope_append_kernel<TI, TO><<<grid, EW_BLOCK, lds, stream>>>(                        \
         (const TI*)qkv, ld, n_tokens, hq, hkv, d, q_gain, k_gain, eps, cos_t, sin_t, rot,       \
         (TO*)q_out, (TO*)kcache, (TO*)vcache, block_table, bt_width, token_seq, token_pos,      \
-        page_size, write_kv)
+        page_size, write_kv, n_splits, split_stride)
     if (in_dtype == ROCML_F32 && out_dtype == ROCML_F32) LAUNCH(float, float);
     else if (in_dtype == ROCML_F32 && out_dtype == ROCML_BF16) LAUNCH(float, bf16_t);
     else if (in_dtype == ROCML_BF16 && out_dtype == ROCML_BF16) LAUNCH(bf16_t, bf16_t);

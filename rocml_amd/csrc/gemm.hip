@@ -36,9 +36,11 @@ static int launch_mfma_tile(const void* x, int ldx, const void* w, int ldw, void
     return 0;
 }
 
+struct SplitPlan { int defer; int* deferred; };
+
 template <int MT, int EPI>
 static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m, int n,
-                         int k, void* workspace, long long workspace_bytes, hipStream_t stream) {
+                         int k, void* workspace, long long workspace_bytes, SplitPlan plan, hipStream_t stream) {
     constexpr int LDS = 2 * MT * 16 * GS_ROW * 16;
     static bool ready = false;
     if (!ready) {
@@ -52,7 +54,7 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
     int by_k = k / 512;
     if (splits > by_k) splits = by_k;
     if (splits > 16) splits = 16;
-    if (splits < 1) splits = 1;
+    if (splits < 1 || EPI == EPI_SWIGLU) splits = 1;     // the gated epilogue needs whole sums
     long long per_split = (long long)m * n * sizeof(float);
     if (splits > 1 && (long long)splits * per_split > workspace_bytes)
         splits = workspace ? (int)(workspace_bytes / per_split) : 1;
@@ -66,6 +68,11 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
     } else {
         gemm_skinny_kernel<MT, EPI, true><<<grid, GS_THREADS, LDS, stream>>>(
             (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, workspace, n, m, n, k, k_per_split);
+        if (plan.defer && ldo == n) {
+            // the caller's next kernel adds the partial sums itself
+            *plan.deferred = splits;
+            return 0;
+        }
         long long total = (long long)m * n;
         gemm_splitk_reduce_kernel<EPI><<<ceil_div(total, 256), 256, 0, stream>>>(
             (const float*)workspace, out, ldo, m, n, splits);
@@ -75,54 +82,114 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
 
 template <int EPI>
 static int launch_skinny_m(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m, int n,
-                           int k, void* workspace, long long workspace_bytes, hipStream_t stream) {
-    if (m <= 16) return launch_skinny<1, EPI>(x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, stream);
-    if (m <= 32) return launch_skinny<2, EPI>(x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, stream);
-    return launch_skinny<4, EPI>(x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, stream);
+                           int k, void* workspace, long long workspace_bytes, SplitPlan plan, hipStream_t stream) {
+    if (m <= 16) return launch_skinny<1, EPI>(x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
+    if (m <= 32) return launch_skinny<2, EPI>(x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
+    return launch_skinny<4, EPI>(x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
+}
+
+// Gated activation over a 32-bit [M, N] product with (gate, up) column pairs: the unfused path of
+// the epilogue above, for the kernels that cannot fuse it.
+template <typename TO>
+__global__ void swiglu_pairs_kernel(const float* __restrict__ gu, TO* __restrict__ out, int ldo, int m, int half) {
+    long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (long long)m * half) return;
+    int r = (int)(idx / half), j = (int)(idx - (long long)r * half);
+    const float* row = gu + (size_t)r * 2 * half;
+    Elem<TO>::store(out + (size_t)r * ldo + j, silu_mul(row[2 * j], row[2 * j + 1]));
+}
+
+// out (+)= sum of split-K partial sums [splits][M][N] in split order: the step that a deferred
+// product leaves to its caller, as a kernel of its own.
+ROCML_EXPORT int rocml_splitk_reduce(const float* partials, void* out, int out_dtype, int ldo, int m, int n,
+                                     int splits, int accumulate, hipStream_t stream) {
+    ROCML_REQUIRE(m >= 0 && n > 0 && splits > 0 && ldo >= n, "splitk_reduce: bad sizes M=%d N=%d splits=%d", m, n, splits);
+    ROCML_REQUIRE(!accumulate || out_dtype == ROCML_F32, "splitk_reduce: accumulation needs a 32-bit output");
+    if (m == 0) return 0;
+    int grid = ceil_div((long long)m * n, 256);
+    if (accumulate) gemm_splitk_reduce_kernel<EPI_ACC><<<grid, 256, 0, stream>>>(partials, out, ldo, m, n, splits);
+    else if (out_dtype == ROCML_F32) gemm_splitk_reduce_kernel<EPI_F32><<<grid, 256, 0, stream>>>(partials, out, ldo, m, n, splits);
+    else if (out_dtype == ROCML_BF16) gemm_splitk_reduce_kernel<EPI_BF16><<<grid, 256, 0, stream>>>(partials, out, ldo, m, n, splits);
+    else return rocml_fail("splitk_reduce: unknown output type %d", out_dtype);
+    ROCML_CHECK_LAUNCH("splitk_reduce");
+    return 0;
 }
 
 // algo: 0 = choose, 1 = plain tiled kernel, 2 = MFMA tile kernel, 3 = MFMA few-rows kernel (M <= 64).
 // accumulate: out += product (out must be 32-bit); this is the residual sum's epilogue.
+// epilogue: 0 = none; 1 = gated activation: W's rows are (gate_j, up_j) pairs and out is
+//   [M, N/2] = silu(gate) * up.
+// defer: if the product was split along K, leave the partial sums [splits][M][N] at the start of
+//   the workspace and report their number in *deferred_splits (0 if the product is complete);
+//   the caller's next kernel adds them.  Needs a dense out (ldo == N).
 // workspace: device memory for split-K partial sums (may be null: no split).
 ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, int w_dtype, int ldw,
                             void* out, int out_dtype, int ldo, int m, int n, int k, int accumulate,
-                            int algo, void* workspace, long long workspace_bytes,
-                            hipStream_t stream) {
+                            int algo, int epilogue, int defer, int* deferred_splits, void* workspace,
+                            long long workspace_bytes, hipStream_t stream) {
+    if (deferred_splits) *deferred_splits = 0;
     ROCML_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm: bad sizes M=%d N=%d K=%d", m, n, k);
-    ROCML_REQUIRE(ldx >= k && ldw >= k && ldo >= n, "gemm: row strides (%d, %d, %d) below (K, K, N)",
+    bool gated = epilogue == 1;
+    ROCML_REQUIRE(epilogue == 0 || epilogue == 1, "gemm: unknown epilogue %d", epilogue);
+    ROCML_REQUIRE(!gated || (n % 2 == 0 && !accumulate), "gemm: the gated epilogue needs an even N and no accumulation");
+    int out_cols = gated ? n / 2 : n;
+    ROCML_REQUIRE(ldx >= k && ldw >= k && ldo >= out_cols, "gemm: row strides (%d, %d, %d) below (K, K, N)",
                   ldx, ldw, ldo);
     ROCML_REQUIRE(!accumulate || out_dtype == ROCML_F32, "gemm: accumulation needs a 32-bit output");
     ROCML_REQUIRE(algo >= ALGO_AUTO && algo <= ALGO_MFMA_SKINNY, "gemm: unknown algorithm %d", algo);
+    ROCML_REQUIRE(!defer || deferred_splits, "gemm: deferring needs a place to report the splits");
     if (m == 0) return 0;
     bool bf16_in = x_dtype == ROCML_BF16 && w_dtype == ROCML_BF16;
     bool mfma_ok = bf16_in && k % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 &&
-                   ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
+                   ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0) && (!gated || out_dtype == ROCML_BF16);
     if (algo >= ALGO_MFMA_TILE)
         ROCML_REQUIRE(mfma_ok, "gemm: the MFMA kernels need bfloat16 operands, K and row strides that are "
                                "multiples of 8 and 16-byte aligned pointers (K=%d ldx=%d ldw=%d)", k, ldx, ldw);
     if (algo == ALGO_MFMA_SKINNY)
         ROCML_REQUIRE(m <= 64, "gemm: the few-rows kernel takes at most 64 rows, got %d", m);
-    int epi = accumulate ? EPI_ACC : (out_dtype == ROCML_BF16 ? EPI_BF16 : EPI_F32);
     ROCML_REQUIRE(out_dtype == ROCML_F32 || out_dtype == ROCML_BF16, "gemm: unknown output type %d", out_dtype);
+    int epi = gated ? EPI_SWIGLU : accumulate ? EPI_ACC : (out_dtype == ROCML_BF16 ? EPI_BF16 : EPI_F32);
     bool use_mfma = mfma_ok && algo != ALGO_PLAIN;
     if (use_mfma) {
         bool skinny = algo == ALGO_MFMA_SKINNY || (algo == ALGO_AUTO && m <= 64);
+        SplitPlan plan{defer, deferred_splits};
         int rc;
 #define BY_EPI(fn, ...)                                              \
         (epi == EPI_F32 ? fn<EPI_F32>(__VA_ARGS__)                   \
-         : epi == EPI_BF16 ? fn<EPI_BF16>(__VA_ARGS__) : fn<EPI_ACC>(__VA_ARGS__))
-        if (skinny) rc = BY_EPI(launch_skinny_m, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, stream);
+         : epi == EPI_BF16 ? fn<EPI_BF16>(__VA_ARGS__)               \
+         : epi == EPI_ACC ? fn<EPI_ACC>(__VA_ARGS__) : fn<EPI_SWIGLU>(__VA_ARGS__))
+        if (skinny) rc = BY_EPI(launch_skinny_m, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
         else rc = BY_EPI(launch_mfma_tile, x, ldx, w, ldw, out, ldo, m, n, k, stream);
 #undef BY_EPI
         if (rc) return rc;
-    } else if (x_dtype == ROCML_F32 && w_dtype == ROCML_F32 && out_dtype == ROCML_F32) {
-        launch_gemm_tile<float, float, float>(x, ldx, w, ldw, out, ldo, m, n, k, accumulate, stream);
-    } else if (bf16_in && out_dtype == ROCML_F32) {
-        launch_gemm_tile<bf16_t, bf16_t, float>(x, ldx, w, ldw, out, ldo, m, n, k, accumulate, stream);
-    } else if (bf16_in && out_dtype == ROCML_BF16) {
-        launch_gemm_tile<bf16_t, bf16_t, bf16_t>(x, ldx, w, ldw, out, ldo, m, n, k, 0, stream);
+        ROCML_CHECK_LAUNCH("gemm");
+        return 0;
+    }
+    // plain kernel; the gated epilogue runs as a second kernel over a 32-bit product in the workspace
+    void* dst = out;
+    int dst_ld = ldo, dst_dtype = out_dtype;
+    if (gated) {
+        ROCML_REQUIRE(workspace && workspace_bytes >= (long long)m * n * (long long)sizeof(float),
+                      "gemm: the gated epilogue needs %lld bytes of workspace", (long long)m * n * 4);
+        dst = workspace;
+        dst_ld = n;
+        dst_dtype = ROCML_F32;
+    }
+    if (x_dtype == ROCML_F32 && w_dtype == ROCML_F32 && dst_dtype == ROCML_F32) {
+        launch_gemm_tile<float, float, float>(x, ldx, w, ldw, dst, dst_ld, m, n, k, accumulate, stream);
+    } else if (bf16_in && dst_dtype == ROCML_F32) {
+        launch_gemm_tile<bf16_t, bf16_t, float>(x, ldx, w, ldw, dst, dst_ld, m, n, k, accumulate, stream);
+    } else if (bf16_in && dst_dtype == ROCML_BF16) {
+        launch_gemm_tile<bf16_t, bf16_t, bf16_t>(x, ldx, w, ldw, dst, dst_ld, m, n, k, 0, stream);
     } else {
         return rocml_fail("gemm: unsupported type triple x=%d w=%d out=%d", x_dtype, w_dtype, out_dtype);
+    }
+    if (gated) {
+        long long total = (long long)m * (n / 2);
+        if (out_dtype == ROCML_F32)
+            swiglu_pairs_kernel<float><<<ceil_div(total, 256), 256, 0, stream>>>((const float*)dst, (float*)out, ldo, m, n / 2);
+        else
+            swiglu_pairs_kernel<bf16_t><<<ceil_div(total, 256), 256, 0, stream>>>((const float*)dst, (bf16_t*)out, ldo, m, n / 2);
     }
     ROCML_CHECK_LAUNCH("gemm");
     return 0;

@@ -35,13 +35,18 @@ __device__ __forceinline__ uint4 load16_or_zero(const bf16_t* p, bool ok) {
     return v;
 }
 
-enum GemmEpilogue : int { EPI_F32 = 0, EPI_BF16 = 1, EPI_ACC = 2 };
+// EPI_SWIGLU: weight rows come in pairs (gate_j, up_j); the output is bfloat16 [M, N/2] with
+// out[m][j] = silu(gate) * up (rocml-kernels/kernels/silu_mul.hip:12-20), formed from the 32-bit
+// accumulators so that gate and up are never rounded or written.
+enum GemmEpilogue : int { EPI_F32 = 0, EPI_BF16 = 1, EPI_ACC = 2, EPI_SWIGLU = 3 };
+
+__device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
 
 template <int EPI>
 __device__ __forceinline__ void epilogue_store(void* out, size_t idx, float v) {
     if (EPI == EPI_F32) ((float*)out)[idx] = v;
     else if (EPI == EPI_BF16) ((bf16_t*)out)[idx] = f32_to_bf16(v);
-    else ((float*)out)[idx] += v;
+    else if (EPI == EPI_ACC) ((float*)out)[idx] += v;
 }
 
 // ---- many rows ---------------------------------------------------------------------------
@@ -131,7 +136,14 @@ gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 int gm = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-                if (gm < m && gn < n) epilogue_store<EPI>(out, (size_t)gm * ldo + gn, acc[i][j][e]);
+                if (EPI == EPI_SWIGLU) {
+                    // neighbouring lanes hold neighbouring columns: the even one has the gate
+                    float other = __shfl_xor(acc[i][j][e], 1, 64);
+                    if ((lane & 1) == 0 && gm < m && gn + 1 < n)
+                        ((bf16_t*)out)[(size_t)gm * ldo + (gn >> 1)] = f32_to_bf16(silu_mul(acc[i][j][e], other));
+                } else if (gm < m && gn < n) {
+                    epilogue_store<EPI>(out, (size_t)gm * ldo + gn, acc[i][j][e]);
+                }
             }
         }
 }
@@ -232,6 +244,16 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restri
     for (int mt = 0; mt < MT; ++mt) {
         int gm = mt * 16 + (lane & 15);
         if (gm >= m) continue;
+        if (EPI == EPI_SWIGLU && !PARTIAL) {
+            // a lane holds weight rows 4g .. 4g+3 = two (gate, up) pairs
+#pragma unroll
+            for (int e = 0; e < 4; e += 2) {
+                int gn = n0 + (lane >> 4) * 4 + e;
+                if (gn + 1 < n)
+                    ((bf16_t*)out)[(size_t)gm * ldo + (gn >> 1)] = f32_to_bf16(silu_mul(acc[mt][e], acc[mt][e + 1]));
+            }
+            continue;
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             int gn = n0 + (lane >> 4) * 4 + e;

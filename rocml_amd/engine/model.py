@@ -90,6 +90,7 @@ class DecoderModel:
         ``[n_want, vocab]`` for the token rows in ``want_rows`` (None if none are wanted)."""
         s = self.spec
         ws = step.workspace
+        ws.drop_pending()
         x = ws.get("model.x", (step.n_tokens, s.hidden), torch.float32)
         ops.embed_gather(self.embed, step.token_ids, x, s.embed_scale)
         for i, entry in enumerate(s.schedule):
@@ -105,9 +106,14 @@ class DecoderModel:
                                          slots=step.seq_slots)
             self.blocks[entry.layer].forward(step, x, view, owner == i)
         if n_want == 0:
+            ws.drop_pending()
             return None
         xn = ws.get("model.final_xn", (n_want, s.hidden), self.dtype)
-        self.final_norm.forward(x, xn, rows=want_rows)
+        if getattr(self.final_norm, "fuses_pending", False):
+            self.final_norm.forward(x, xn, rows=want_rows, pending=ws.take_pending(x))
+        else:
+            ws.flush_pending()
+            self.final_norm.forward(x, xn, rows=want_rows)
         logits = ws.get("model.logits", (n_want, s.vocab), torch.float32)
         ops.gemm(xn, self.lm_head, logits, workspace=ws.scratch())
         return logits

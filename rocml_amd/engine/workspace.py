@@ -23,6 +23,7 @@ class Workspace:
         self.generation = 0
         self._scratch_bytes = scratch_bytes
         self._scratch = None
+        self._pending = None
 
     def get(self, name: str, shape: Tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
         n = math.prod(shape)
@@ -35,11 +36,50 @@ class Workspace:
         return buf[:n].view(shape)
 
     def scratch(self) -> torch.Tensor:
-        """Device memory kernels may use for partial results of one launch."""
+        """Device memory kernels may use for partial results of one launch.  Partial sums
+        that a deferred product left there are added to their target first."""
         if self._scratch is None:
             self._scratch = torch.empty(self._scratch_bytes, dtype=torch.uint8, device=self.device)
             self.generation += 1
+        self.flush_pending()
         return self._scratch
+
+    # -- deferred split-K sums --------------------------------------------------------------
+    # A product that was split along K and whose result is to be added to a tensor may leave
+    # its partial sums in the scratch memory; the next kernel that reads the tensor (a norm)
+    # adds them itself.  Whoever needs the scratch memory or the tensor before that calls
+    # flush_pending, which runs the addition as a kernel of its own.
+    def set_pending(self, target: torch.Tensor, n_splits: int) -> None:
+        self.flush_pending()
+        self._pending = (target, n_splits)
+
+    def _partials(self) -> torch.Tensor:
+        target, n_splits = self._pending
+        n = n_splits * target.numel()
+        return self._scratch[:n * 4].view(torch.float32).view(n_splits, target.shape[0], target.shape[1])
+
+    def take_pending(self, target: torch.Tensor):
+        """The partial sums waiting for ``target`` (``[splits, rows, n]``), which the caller
+        now adds itself; None if there are none."""
+        if self._pending is None:
+            return None
+        if self._pending[0].data_ptr() != target.data_ptr():
+            self.flush_pending()
+            return None
+        partials = self._partials()
+        self._pending = None
+        return partials
+
+    def flush_pending(self) -> None:
+        if self._pending is not None:
+            from .. import ops
+            partials = self._partials()
+            target = self._pending[0]
+            self._pending = None
+            ops.splitk_reduce(partials, target, accumulate=True)
+
+    def drop_pending(self) -> None:
+        self._pending = None
 
     def bytes(self) -> int:
         total = sum(b.numel() * b.element_size() for b in self._buffers.values())

@@ -28,15 +28,16 @@ _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 _SIGNATURES = {
     "elementwise": {
         "rocml_embed_gather": [_P, _I, _P, _P, _I, _I, _I, _F, _P],
-        "rocml_rmsnorm": [_P, _P, _P, _I, _P, _I, _I, _F, _P],
-        "rocml_swiglu": [_P, _I, _P, _I, _I, _I, _P],
+        "rocml_rmsnorm": [_P, _P, _P, _I, _P, _I, _I, _F, _P, _I, _LL, _P],
+        "rocml_swiglu": [_P, _I, _P, _I, _I, _I, _I, _P],
         "rocml_rope_table": [_P, _P, _P, _P, _I, _I, _P],
         "rocml_qk_norm_rope_append": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P, _P, _I, _P, _P, _P,
-                                      _I, _P, _I, _P, _P, _I, _I, _P],
+                                      _I, _P, _I, _P, _P, _I, _I, _I, _LL, _P],
         "rocml_add_into": [_P, _P, _I, _LL, _P],
     },
     "gemm": {
-        "rocml_gemm": [_P, _I, _I, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _LL, _P],
+        "rocml_gemm": [_P, _I, _I, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _LL, _P],
+        "rocml_splitk_reduce": [_P, _P, _I, _I, _I, _I, _I, _I, _P],
     },
     "attention": {
         "rocml_attention": [_P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I,
@@ -131,8 +132,11 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scal
 
 
 def rmsnorm(x: torch.Tensor, gain: torch.Tensor, eps: float, out: torch.Tensor,
-            rows: Optional[torch.Tensor] = None) -> None:
-    _dev(x, gain, out, rows)
+            rows: Optional[torch.Tensor] = None, partials: Optional[torch.Tensor] = None) -> None:
+    """``partials`` ([splits, rows of x, n] float32) are split-K partial sums that belong to
+    ``x``: the kernel adds them to ``x`` first (and stores the sum back unless rows are
+    gathered)."""
+    _dev(x, gain, out, rows, partials)
     _want(x, torch.float32, "norm input")
     _want(gain, torch.float32, "norm gain")
     n = x.shape[-1]
@@ -145,17 +149,26 @@ def rmsnorm(x: torch.Tensor, gain: torch.Tensor, eps: float, out: torch.Tensor,
             raise KernelError("one row index per output row is needed")
     elif x.numel() != out.numel():
         raise KernelError("norm input and output differ in size")
+    n_splits, stride = 0, 0
+    if partials is not None:
+        _want(partials, torch.float32, "partial sums")
+        if partials.dim() != 3 or partials.shape[1] * partials.shape[2] != x.numel():
+            raise KernelError(f"partial sums {tuple(partials.shape)} do not fit the norm input {tuple(x.shape)}")
+        n_splits, stride = partials.shape[0], x.numel()
     _check("elementwise", library("elementwise").rocml_rmsnorm(
-        _ptr(x), _ptr(gain), _ptr(out), _code(out), _ptr(rows), n_rows, n, eps, _stream()))
+        _ptr(x), _ptr(gain), _ptr(out), _code(out), _ptr(rows), n_rows, n, eps, _ptr(partials), n_splits,
+        stride, _stream()))
 
 
-def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor, interleaved: bool = False) -> None:
+    """``gate_up`` rows hold the gate half then the up half, or (gate, up) pairs when
+    ``interleaved``."""
     _dev(gate_up, out)
     n_tokens, inter = out.shape
     if gate_up.shape != (n_tokens, 2 * inter):
         raise KernelError(f"gate/up is {tuple(gate_up.shape)}, expected {(n_tokens, 2 * inter)}")
     _check("elementwise", library("elementwise").rocml_swiglu(
-        _ptr(gate_up), _code(gate_up), _ptr(out), _code(out), n_tokens, inter, _stream()))
+        _ptr(gate_up), _code(gate_up), _ptr(out), _code(out), n_tokens, inter, 1 if interleaved else 0, _stream()))
 
 
 def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> None:
@@ -176,11 +189,18 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
                         cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rot_dim: int,
                         q_out: torch.Tensor, k_cache: Optional[torch.Tensor],
                         v_cache: Optional[torch.Tensor], block_table: Optional[torch.Tensor],
-                        token_seq: torch.Tensor, token_pos: torch.Tensor, write_kv: bool = True) -> None:
+                        token_seq: torch.Tensor, token_pos: torch.Tensor, write_kv: bool = True,
+                        n_splits: int = 1) -> None:
     """``qkv`` is ``[T, ld]`` with q, k, v side by side (k and v may be absent when
     ``write_kv`` is false).  Keys are ``[pages, Hkv, page_size, D]``, values
     ``[pages, Hkv, D, page_size]``."""
     _dev(qkv, q_gain, k_gain, cos, sin, q_out, k_cache, v_cache, block_table, token_seq, token_pos)
+    split_stride = 0
+    if n_splits > 1:                      # [splits, T, ld] split-K partial sums, added in the kernel
+        if qkv.dim() != 3 or qkv.shape[0] != n_splits:
+            raise KernelError("partial sums of the projection must be [splits, tokens, width]")
+        split_stride = qkv.shape[1] * qkv.shape[2]
+        qkv = qkv[0]
     n_tokens, ld = qkv.shape
     for g in (q_gain, k_gain):
         if g is not None:
@@ -208,7 +228,7 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
         _ptr(qkv), _code(qkv), ld, n_tokens, n_heads, n_kv_heads, head_dim, _ptr(q_gain), _ptr(k_gain),
         eps, _ptr(cos), _ptr(sin), rot_dim if cos is not None else 0, _ptr(q_out), _ptr(k_cache),
         _ptr(v_cache), _code(q_out), _ptr(block_table), bt_width, _ptr(token_seq), _ptr(token_pos),
-        page_size, 1 if write_kv else 0, _stream()))
+        page_size, 1 if write_kv else 0, n_splits, split_stride, _stream()))
 
 
 def add_into(x: torch.Tensor, y: torch.Tensor) -> None:
@@ -224,23 +244,45 @@ GEMM_AUTO, GEMM_PLAIN = 0, 1
 
 
 def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
-         algo: int = GEMM_AUTO, workspace: Optional[torch.Tensor] = None) -> None:
+         algo: int = GEMM_AUTO, workspace: Optional[torch.Tensor] = None, epilogue: Optional[str] = None,
+         defer: bool = False) -> int:
     """``out (+)= x @ w.T`` for ``x [M, K]``, ``w [N, K]``, ``out [M, N]`` (rows may be
-    strided views with unit inner stride)."""
+    strided views with unit inner stride).  ``epilogue="swiglu"``: ``w``'s rows are (gate, up)
+    pairs and ``out`` is ``[M, N/2] = silu(gate) * up``.  With ``defer`` a product that was
+    split along K leaves its partial sums ``[splits, M, N]`` at the start of ``workspace`` and
+    returns their number for the caller's next kernel to add; it returns 0 when ``out`` is
+    complete."""
     for t in (x, w, out):
         if not t.is_cuda:
             raise KernelError("kernel arguments must be GPU tensors; this library has no CPU path")
         if t.dim() != 2 or t.stride(1) != 1:
             raise KernelError("matrix product operands must be 2-D with unit inner stride")
+    if epilogue not in (None, "swiglu"):
+        raise KernelError(f"unknown epilogue {epilogue!r}")
     m, k = x.shape
     n = w.shape[0]
-    if w.shape[1] != k or out.shape != (m, n):
+    cols = n // 2 if epilogue else n
+    if w.shape[1] != k or out.shape != (m, cols):
         raise KernelError(f"matrix product shapes do not fit: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
     ws_ptr, ws_bytes = (None, 0) if workspace is None else (workspace.data_ptr(), workspace.numel() * workspace.element_size())
+    deferred = ctypes.c_int(0)
     _check("gemm", library("gemm").rocml_gemm(
         _ptr(x), _code(x), x.stride(0) if m > 1 else max(x.stride(0), k), _ptr(w), _code(w), w.stride(0),
-        _ptr(out), _code(out), out.stride(0) if m > 1 else max(out.stride(0), n), m, n, k,
-        1 if accumulate else 0, algo, ws_ptr, ws_bytes, _stream()))
+        _ptr(out), _code(out), out.stride(0) if m > 1 else max(out.stride(0), cols), m, n, k,
+        1 if accumulate else 0, algo, 1 if epilogue else 0, 1 if defer else 0, ctypes.byref(deferred), ws_ptr,
+        ws_bytes, _stream()))
+    return deferred.value
+
+
+def splitk_reduce(partials: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+    """``out (+)= partials.sum(0)`` in split order, for ``partials [splits, M, N]`` float32."""
+    _dev(partials, out)
+    _want(partials, torch.float32, "partial sums")
+    splits, m, n = partials.shape
+    if out.shape != (m, n):
+        raise KernelError("partial sums and output differ in shape")
+    _check("gemm", library("gemm").rocml_splitk_reduce(_ptr(partials), _ptr(out), _code(out), out.stride(0), m, n,
+                                                       splits, 1 if accumulate else 0, _stream()))
 
 
 # ---- attention -----------------------------------------------------------------------

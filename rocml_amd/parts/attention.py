@@ -78,7 +78,10 @@ class Attention(Mixer):
         ws = step.workspace
         rows = self.q_dim + 2 * self.kv_dim if owns_cache else self.q_dim
         qkv = ws.get("attn.qkv", (n, rows), torch.float32)
-        ops.gemm(xn, self.w_qkv[:rows], qkv, workspace=ws.scratch())
+        scratch = ws.scratch()
+        splits = ops.gemm(xn, self.w_qkv[:rows], qkv, workspace=scratch, defer=True)
+        if splits:      # the product's split-K partial sums; the next kernel adds them
+            qkv = scratch[:splits * n * rows * 4].view(torch.float32).view(splits, n, rows)
         cos = sin = None
         rot = 0
         if self.position is not None:
@@ -88,13 +91,15 @@ class Attention(Mixer):
         eps = s.qk_norm.eps if s.qk_norm is not None else 1.0
         ops.qk_norm_rope_append(qkv, s.n_heads, s.n_kv_heads, s.head_dim, self.q_gain, self.k_gain, eps,
                                 cos, sin, rot, q, cache.k, cache.v, cache.block_table, step.token_seq,
-                                step.token_pos, write_kv=owns_cache)
+                                step.token_pos, write_kv=owns_cache, n_splits=max(splits, 1))
         o = ws.get("attn.o", (n, self.q_dim), self.dtype)
         ops.attention(q, o, cache.k, cache.v, cache.block_table, step.token_seq, step.token_pos,
                       s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, workspace=ws.scratch(),
                       cu_seqlens=step.cu_seqlens, max_new=step.max_new, total_q_tiles=step.total_q_tiles,
                       max_len=step.max_len, n_splits=self._decode_splits(step, cache))
-        ops.gemm(o, self.w_o, x_accum, accumulate=True, workspace=ws.scratch())
+        splits = ops.gemm(o, self.w_o, x_accum, accumulate=True, workspace=ws.scratch(), defer=True)
+        if splits:
+            ws.set_pending(x_accum, splits)
 
 
 register_mixer("attention", Attention)

@@ -13,7 +13,10 @@ layer is assembled from parts that know nothing about the model around them:
 * a **position encoding** prepares per-step tables that mixers share.
 
 Mixers and feed-forwards add their result into the 32-bit residual stream they are
-handed (``x_accum``), which lets a product's epilogue do the residual sum.
+handed (``x_accum``), which lets a product's epilogue do the residual sum.  A part whose
+last product was split along K may leave the final addition of the partial sums to the
+norm that reads ``x_accum`` next (``step.workspace.set_pending``); whoever reads
+``x_accum`` in another way calls ``step.workspace.flush_pending()`` first.
 """
 from __future__ import annotations
 

@@ -40,10 +40,21 @@ class PreNormBlock(Part):
 
     def forward(self, step, x: torch.Tensor, cache, owns_cache: bool) -> None:
         xn = step.workspace.get("block.xn", tuple(x.shape), self.dtype)
-        self.mixer_norm.forward(x, xn)
+        self._norm(step, self.mixer_norm, x, xn)
         self.mixer.forward(step, xn, x, cache, owns_cache)
-        self.ffn_norm.forward(x, xn)
+        self._norm(step, self.ffn_norm, x, xn)
         self.ffn.forward(step, xn, x)
+
+    @staticmethod
+    def _norm(step, norm, x, xn) -> None:
+        """A part may leave the last step of its residual sum (adding split-K partial sums
+        to x) to the norm that reads x next; a norm that cannot do that gets x completed."""
+        ws = step.workspace
+        if getattr(norm, "fuses_pending", False):
+            norm.forward(x, xn, pending=ws.take_pending(x))
+        else:
+            ws.flush_pending()
+            norm.forward(x, xn)
 
 
 register_block("pre_norm", PreNormBlock)

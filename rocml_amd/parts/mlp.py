@@ -31,18 +31,27 @@ class GatedMlp(FeedForward):
                 "down_proj.weight": ParamSpec((s.hidden, s.intermediate))}
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.w_gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]], dim=0).contiguous()
+        # Rows in (gate_j, up_j) pairs: the product's epilogue then has both halves of an
+        # output in one lane and applies the activation to its 32-bit sums.
+        gate, up = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        self.w_gate_up = torch.stack([gate, up], dim=1).reshape(2 * gate.shape[0], gate.shape[1]).contiguous()
         self.w_down = tensors["down_proj.weight"]
+        self.fused = self.dtype == torch.bfloat16 and self.spec.hidden % 8 == 0
 
     def forward(self, step, xn, x_accum) -> None:
         s = self.spec
         n = step.n_tokens
         ws = step.workspace
-        gate_up = ws.get("mlp.gate_up", (n, 2 * s.intermediate), torch.float32)
-        ops.gemm(xn, self.w_gate_up, gate_up, workspace=ws.scratch())
         h = ws.get("mlp.h", (n, s.intermediate), self.dtype)
-        ops.swiglu(gate_up, h)
-        ops.gemm(h, self.w_down, x_accum, accumulate=True, workspace=ws.scratch())
+        if self.fused:
+            ops.gemm(xn, self.w_gate_up, h, workspace=ws.scratch(), epilogue="swiglu")
+        else:
+            gate_up = ws.get("mlp.gate_up", (n, 2 * s.intermediate), torch.float32)
+            ops.gemm(xn, self.w_gate_up, gate_up, workspace=ws.scratch())
+            ops.swiglu(gate_up, h, interleaved=True)
+        splits = ops.gemm(h, self.w_down, x_accum, accumulate=True, workspace=ws.scratch(), defer=True)
+        if splits:
+            ws.set_pending(x_accum, splits)
 
 
 register_feed_forward("gated_mlp", GatedMlp)

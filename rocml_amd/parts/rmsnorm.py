@@ -25,8 +25,11 @@ class RMSNorm(Norm):
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.gain = tensors["weight"]
 
-    def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
-        ops.rmsnorm(x, self.gain, self.eps, out, rows)
+    fuses_pending = True      # forward() can add a deferred product's partial sums to x itself
+
+    def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None,
+                pending: Optional[torch.Tensor] = None) -> None:
+        ops.rmsnorm(x, self.gain, self.eps, out, rows, partials=pending)
 
 
 register_norm("rmsnorm", RMSNorm)

@@ -45,6 +45,26 @@ def test_rmsnorm(rows, n):
         assert float((got.cpu().double() - want[[rows - 1, 0, rows - 1]]).abs().max()) < 1e-5
 
 
+@pytest.mark.parametrize("rows,n,splits", [(3, 4096, 8), (2, 96, 3), (5, 300, 1), (1, 30, 5)])
+def test_rmsnorm_adds_partial_sums(rows, n, splits):
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(rows, n, generator=g)
+    w = 1 + 0.1 * torch.randn(n, generator=g)
+    partials = torch.randn(splits, rows, n, generator=g)
+    total = x.double() + partials.double().sum(0)
+    want = plain.rmsnorm(total, w.double(), 1e-5)
+    xd, out = x.cuda(), torch.empty(rows, n, device="cuda")
+    ops.rmsnorm(xd, w.cuda(), 1e-5, out, partials=partials.cuda())
+    assert float((out.cpu().double() - want).abs().max()) < 1e-5
+    assert float((xd.cpu().double() - total).abs().max()) < 1e-5          # the sum went back into x
+    xd = x.cuda()
+    idx = torch.tensor([rows - 1, rows - 1, 0], dtype=torch.int32).cuda()
+    got = torch.empty(3, n, device="cuda")
+    ops.rmsnorm(xd, w.cuda(), 1e-5, got, rows=idx, partials=partials.cuda())
+    assert float((got.cpu().double() - want[[rows - 1, rows - 1, 0]]).abs().max()) < 1e-5
+    assert torch.equal(xd.cpu(), x)                                       # gathered rows: x is left alone
+
+
 @pytest.mark.parametrize("tokens,inter", [(1, 1000), (1, 1), (7, 33)])
 def test_swiglu(tokens, inter):
     n = tokens * inter
@@ -58,6 +78,9 @@ def test_swiglu(tokens, inter):
     out16 = torch.empty(tokens, inter, dtype=torch.bfloat16, device="cuda")
     ops.swiglu(gu, out16)
     assert float((out16.cpu().double() - want).abs().max()) < 8e-3 * max(1.0, float(want.abs().max()))
+    pairs = torch.stack([gate, up], dim=2).reshape(tokens, 2 * inter).cuda()
+    ops.swiglu(pairs, out, interleaved=True)
+    assert float((out.cpu().double() - want).abs().max()) < 1e-6
 
 
 def test_add_into():
@@ -72,7 +95,7 @@ def test_add_into():
     assert torch.equal(x, want)
 
 
-def _qkv_case(tokens, hq, hkv, d, pos_base, theta, rot, norm, dtype, seed=0):
+def _qkv_case(tokens, hq, hkv, d, pos_base, theta, rot, norm, dtype, seed=0, splits=1):
     """Runs the fused kernel on one sequence whose pages are handed out backwards; returns
     (q, k rows, v rows) read back from q_out and the cache, and the plain expectation."""
     g = torch.Generator().manual_seed(seed)
@@ -95,10 +118,16 @@ def _qkv_case(tokens, hq, hkv, d, pos_base, theta, rot, norm, dtype, seed=0):
         cos = torch.empty(tokens, rot // 2, device="cuda")
         sin = torch.empty(tokens, rot // 2, device="cuda")
         ops.rope_table(torch.tensor(positions, dtype=torch.int32).cuda(), inv, cos, sin)
-    ops.qk_norm_rope_append(qkv.cuda(), hq, hkv, d, qg.cuda() if norm else None, kg.cuda() if norm else None, eps,
+    fed = qkv.cuda()
+    if splits > 1:                      # the same values as a sum of parts
+        parts = torch.randn(splits, tokens, ld, generator=g)
+        parts[0] = qkv - parts[1:].sum(0)
+        qkv = parts.sum(0)
+        fed = parts.cuda()
+    ops.qk_norm_rope_append(fed, hq, hkv, d, qg.cuda() if norm else None, kg.cuda() if norm else None, eps,
                             cos, sin, rot, q_out, kc, vc, table.cuda(),
                             torch.zeros(tokens, dtype=torch.int32).cuda(),
-                            torch.tensor(positions, dtype=torch.int32).cuda())
+                            torch.tensor(positions, dtype=torch.int32).cuda(), n_splits=splits)
     q = qkv[:, :hq * d].reshape(tokens, hq, d).double()
     k = qkv[:, hq * d:(hq + hkv) * d].reshape(tokens, hkv, d).double()
     v = qkv[:, (hq + hkv) * d:].reshape(tokens, hkv, d).double()
@@ -129,6 +158,12 @@ def test_qk_norm_rope_append(tokens, hq, hkv, d, pos_base, rot, norm):
     assert float((gq - q).abs().max()) < 8e-3 * float(q.abs().max())
     assert float((gk - k).abs().max()) < 8e-3 * float(k.abs().max())
     assert float((gv - _bf16(v)).abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("splits", [2, 5, 8])
+def test_qk_norm_rope_append_adds_partial_sums(splits):
+    gq, gk, gv, q, k, v, _ = _qkv_case(9, 4, 2, 128, 60, 1e4, 128, True, torch.float32, splits=splits)
+    assert float((gq - q).abs().max()) < 2e-5 and float((gk - k).abs().max()) < 2e-5 and float((gv - v).abs().max()) < 2e-6
 
 
 def test_rotation_table_at_large_positions():

@@ -77,3 +77,43 @@ def test_strided_rows_and_refusals():
         ops.gemm(odd, w2, out2, algo=TILE)
     with pytest.raises(KernelError):
         ops.gemm(x.cpu(), w, out)
+
+
+@pytest.mark.parametrize("algo", [PLAIN, TILE, SKINNY])
+@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (7, 448, 96), (64, 1000, 264), (130, 256, 128), (300, 2048, 512)])
+def test_gated_epilogue(m, n, k, algo):
+    """Rows of the weight are (gate, up) pairs; the output is silu(gate) * up, formed from
+    the 32-bit sums."""
+    if algo == SKINNY and m > 64:
+        pytest.skip("the few-rows kernel takes at most 64 rows")
+    x, w = _operands(m, n, k, torch.bfloat16, 3)
+    full = _ref(x, w)
+    gate, up = full[:, 0::2], full[:, 1::2]
+    ref = gate / (1 + torch.exp(-gate)) * up
+    ws = torch.empty(16 << 20, dtype=torch.uint8, device="cuda")
+    out = torch.empty(m, n // 2, dtype=torch.bfloat16, device="cuda")
+    ops.gemm(x, w, out, algo=algo, workspace=ws, epilogue="swiglu")
+    assert float((out.double().cpu() - ref.cpu()).abs().max()) < 5e-3 * max(1.0, float(ref.abs().max()))
+    if algo == PLAIN:
+        x32, w32 = x.float(), w.float()
+        out32 = torch.empty(m, n // 2, dtype=torch.float32, device="cuda")
+        ops.gemm(x32, w32, out32, workspace=ws, epilogue="swiglu")
+        assert float((out32.double().cpu() - ref.cpu()).abs().max()) < 2e-5 * max(1.0, float(ref.abs().max()))
+
+
+def test_deferred_split_sums():
+    """A product split along K may leave its partial sums to the caller; adding them in split
+    order gives the product."""
+    x, w = _operands(8, 256, 4096, torch.bfloat16, 4)
+    ref = _ref(x, w)
+    ws = torch.empty(16 << 20, dtype=torch.uint8, device="cuda")
+    base = torch.randn(8, 256, device="cuda")
+    out = base.clone()
+    splits = ops.gemm(x, w, out, accumulate=True, workspace=ws, defer=True)
+    assert splits > 1 and torch.equal(out, base)              # nothing was added yet
+    partials = ws[:splits * 8 * 256 * 4].view(torch.float32).view(splits, 8, 256)
+    assert float((partials.double().sum(0) - ref).abs().max()) < 2e-5 * float(ref.abs().max())
+    ops.splitk_reduce(partials, out, accumulate=True)
+    assert float((out.double() - (ref + base.double())).abs().max()) < 2e-5 * float(ref.abs().max())
+    assert ops.gemm(x, w, out, workspace=None, defer=True) == 0   # no workspace: no split, complete result
+    assert float((out.double() - ref).abs().max()) < 2e-5 * float(ref.abs().max())

@@ -146,6 +146,7 @@ def test_norm_rope_and_mlp_parts_alone():
                        seq_slots=pos, max_new=9, max_len=9, total_q_tiles=1, workspace=Workspace("cuda:0"))
     acc = x.cuda().clone()
     ffn.forward(step, x.cuda(), acc)
+    step.workspace.flush_pending()                                       # a part may leave its last sum to the next norm
     xd = x.double()
     want = xd + plain.swiglu(xd @ ws["gate_proj.weight"].double().t(), xd @ ws["up_proj.weight"].double().t()) \
         @ ws["down_proj.weight"].double().t()
