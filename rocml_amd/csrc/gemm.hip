@@ -8,7 +8,7 @@
 
 ROCML_LAST_ERROR_FN(gemm)
 
-enum GemmAlgo : int { ALGO_AUTO = 0, ALGO_PLAIN = 1, ALGO_MFMA_TILE = 2, ALGO_MFMA_SKINNY = 3 };
+enum GemmAlgo : int { ALGO_AUTO = 0, ALGO_PLAIN = 1, ALGO_MFMA_TILE = 2, ALGO_MFMA_SKINNY = 3, ALGO_MFMA_KPAR = 4 };
 
 static int round_up(int a, int b) { return (a + b - 1) / b * b; }
 
@@ -80,6 +80,41 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
     return 0;
 }
 
+// At most 16 rows: blocks of 16 weight rows, K split over the block's waves and, while there are
+// fewer than about 1000 blocks, over blocks as well (each wave keeps at least 256 of K).
+template <int EPI>
+static int launch_kpar(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m, int n, int k,
+                       void* workspace, long long workspace_bytes, SplitPlan plan, hipStream_t stream) {
+    int n_tiles = ceil_div(n, 16);
+    int splits = 1024 / n_tiles;
+    int by_k = k / 1024;
+    if (splits > by_k) splits = by_k;
+    if (splits > 16) splits = 16;
+    if (splits < 1 || EPI == EPI_SWIGLU) splits = 1;
+    long long per_split = (long long)m * n * sizeof(float);
+    if (splits > 1 && (long long)splits * per_split > workspace_bytes)
+        splits = workspace ? (int)(workspace_bytes / per_split) : 1;
+    if (splits < 1) splits = 1;
+    int k_per_split = round_up(ceil_div(k, splits), 128);
+    splits = ceil_div(k, k_per_split);
+    dim3 grid(n_tiles, splits);
+    if (splits == 1) {
+        gemm_kpar_kernel<EPI, false><<<grid, GK_THREADS, 0, stream>>>(
+            (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
+    } else {
+        gemm_kpar_kernel<EPI, true><<<grid, GK_THREADS, 0, stream>>>(
+            (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, workspace, n, m, n, k, k_per_split);
+        if (plan.defer && ldo == n) {
+            *plan.deferred = splits;
+            return 0;
+        }
+        long long total = (long long)m * n;
+        gemm_splitk_reduce_kernel<EPI><<<ceil_div(total, 256), 256, 0, stream>>>(
+            (const float*)workspace, out, ldo, m, n, splits);
+    }
+    return 0;
+}
+
 template <int EPI>
 static int launch_skinny_m(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m, int n,
                            int k, void* workspace, long long workspace_bytes, SplitPlan plan, hipStream_t stream) {
@@ -115,7 +150,8 @@ ROCML_EXPORT int rocml_splitk_reduce(const float* partials, void* out, int out_d
     return 0;
 }
 
-// algo: 0 = choose, 1 = plain tiled kernel, 2 = MFMA tile kernel, 3 = MFMA few-rows kernel (M <= 64).
+// algo: 0 = choose, 1 = plain tiled kernel, 2 = MFMA tile kernel, 3 = MFMA few-rows kernel (M <= 64),
+// 4 = MFMA kernel for at most 16 rows.
 // accumulate: out += product (out must be 32-bit); this is the residual sum's epilogue.
 // epilogue: 0 = none; 1 = gated activation: W's rows are (gate_j, up_j) pairs and out is
 //   [M, N/2] = silu(gate) * up.
@@ -136,7 +172,7 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
     ROCML_REQUIRE(ldx >= k && ldw >= k && ldo >= out_cols, "gemm: row strides (%d, %d, %d) below (K, K, N)",
                   ldx, ldw, ldo);
     ROCML_REQUIRE(!accumulate || out_dtype == ROCML_F32, "gemm: accumulation needs a 32-bit output");
-    ROCML_REQUIRE(algo >= ALGO_AUTO && algo <= ALGO_MFMA_SKINNY, "gemm: unknown algorithm %d", algo);
+    ROCML_REQUIRE(algo >= ALGO_AUTO && algo <= ALGO_MFMA_KPAR, "gemm: unknown algorithm %d", algo);
     ROCML_REQUIRE(!defer || deferred_splits, "gemm: deferring needs a place to report the splits");
     if (m == 0) return 0;
     bool bf16_in = x_dtype == ROCML_BF16 && w_dtype == ROCML_BF16;
@@ -147,6 +183,8 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
                                "multiples of 8 and 16-byte aligned pointers (K=%d ldx=%d ldw=%d)", k, ldx, ldw);
     if (algo == ALGO_MFMA_SKINNY)
         ROCML_REQUIRE(m <= 64, "gemm: the few-rows kernel takes at most 64 rows, got %d", m);
+    if (algo == ALGO_MFMA_KPAR)
+        ROCML_REQUIRE(m <= 16, "gemm: the 16-rows kernel takes at most 16 rows, got %d", m);
     ROCML_REQUIRE(out_dtype == ROCML_F32 || out_dtype == ROCML_BF16, "gemm: unknown output type %d", out_dtype);
     int epi = gated ? EPI_SWIGLU : accumulate ? EPI_ACC : (out_dtype == ROCML_BF16 ? EPI_BF16 : EPI_F32);
     bool use_mfma = mfma_ok && algo != ALGO_PLAIN;
@@ -158,7 +196,9 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
         (epi == EPI_F32 ? fn<EPI_F32>(__VA_ARGS__)                   \
          : epi == EPI_BF16 ? fn<EPI_BF16>(__VA_ARGS__)               \
          : epi == EPI_ACC ? fn<EPI_ACC>(__VA_ARGS__) : fn<EPI_SWIGLU>(__VA_ARGS__))
-        if (skinny) rc = BY_EPI(launch_skinny_m, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
+        bool kpar = algo == ALGO_MFMA_KPAR || (algo == ALGO_AUTO && m <= 2);   // beyond two rows the activations read from L2 cost more than the block sharing of the few-rows kernel
+        if (kpar) rc = BY_EPI(launch_kpar, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
+        else if (skinny) rc = BY_EPI(launch_skinny_m, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
         else rc = BY_EPI(launch_mfma_tile, x, ldx, w, ldw, out, ldo, m, n, k, stream);
 #undef BY_EPI
         if (rc) return rc;

@@ -264,6 +264,82 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restri
     }
 }
 
+// ---- at most 16 rows -------------------------------------------------------------------------
+// The decode step of a small batch.  A block owns 16 weight rows and a K range; its four waves
+// take a quarter of the range each and never meet before the end: weights and activations go
+// from global memory (the activations are small and stay in L2) straight into MFMA operand
+// registers, two rounds of 8 loads of 16 bytes per lane in flight, no LDS and no barrier in the
+// loop.  With 16 rows per block even the widest projection gives thousands of waves, which is
+// what keeps enough bytes in flight to stream weights at memory speed.  The four partial tiles
+// are added in wave order through LDS, then comes the epilogue (or the split-K partial store).
+constexpr int GK_KC = 256, GK_THREADS = 256;
+
+template <int EPI, bool PARTIAL>
+__global__ void __launch_bounds__(GK_THREADS)
+gemm_kpar_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw,
+                 void* __restrict__ out, int ldo, int m, int n, int k, int k_per_split) {
+    __shared__ float red[4][64][4];
+    int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int g = lane >> 4, col = lane & 15;
+    int tile = blockIdx.x, split = blockIdx.y;
+    int bs = split * k_per_split, be = min(k, bs + k_per_split);
+    int quarter = (((be - bs + 3) / 4) + 31) / 32 * 32;
+    int ks = min(be, bs + wave * quarter), ke = min(be, ks + quarter);
+    int wrow = tile * 16 + col;
+    bool wok = wrow < n, xok = col < m;
+    const bf16_t* wp = w + (size_t)(wok ? wrow : 0) * ldw + g * 8;
+    const bf16_t* xp = x + (size_t)(xok ? col : 0) * ldx + g * 8;
+    uint4 wc[8], xc[8], wn[8], xn[8];
+    f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    auto load = [&](int kb, uint4* wd, uint4* xd) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            int gk = kb + j * 32;
+            bool ok = gk + g * 8 < ke;
+            wd[j] = load16_or_zero(ok ? wp + gk : w, ok && wok);
+            xd[j] = load16_or_zero(ok ? xp + gk : x, ok && xok);
+        }
+    };
+    if (ks < ke) load(ks, wc, xc);
+    for (int kb = ks; kb < ke; kb += GK_KC) {
+        bool more = kb + GK_KC < ke;
+        if (more) load(kb + GK_KC, wn, xn);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(wc[j]), as_frag(xc[j]), acc, 0, 0, 0);
+        if (more) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                wc[j] = wn[j];
+                xc[j] = xn[j];
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) red[wave][lane][e] = acc[e];
+    __syncthreads();
+    if (wave != 0 || !xok) return;
+    float sum[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sum[e] = ((red[0][lane][e] + red[1][lane][e]) + red[2][lane][e]) + red[3][lane][e];
+    // element e of a lane: weight row 4g + e of the tile, activation row lane%16
+    int gn0 = tile * 16 + g * 4;
+    if (EPI == EPI_SWIGLU && !PARTIAL) {
+#pragma unroll
+        for (int e = 0; e < 4; e += 2)
+            if (gn0 + e + 1 < n)
+                ((bf16_t*)out)[(size_t)col * ldo + ((gn0 + e) >> 1)] = f32_to_bf16(silu_mul(sum[e], sum[e + 1]));
+        return;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        int gn = gn0 + e;
+        if (gn >= n) continue;
+        if (PARTIAL) ((float*)out)[((size_t)split * m + col) * n + gn] = sum[e];
+        else epilogue_store<EPI>(out, (size_t)col * ldo + gn, sum[e]);
+    }
+}
+
 // out[m][n] (+)= sum over splits, in split order.
 template <int EPI>
 __global__ void gemm_splitk_reduce_kernel(const float* __restrict__ partial, void* __restrict__ out,

@@ -238,10 +238,59 @@ argmax_kernel(const float* __restrict__ logits, int vocab, int* __restrict__ out
     if (threadIdx.x == 0) out[b] = best.i == 0x7fffffff ? 0 : best.i;
 }
 
-ROCML_EXPORT int rocml_argmax(const float* logits, int batch, int vocab, int* out, hipStream_t stream) {
+// Two stages for long rows: a row is cut into ARGMAX_CHUNKS pieces, each block finds its piece's
+// first maximum, a second kernel picks among the pieces (lower piece wins a tie, so the first
+// maximum of the row wins).  One block per row would read a 150k-entry row alone.
+constexpr int ARGMAX_CHUNKS = 32;
+
+__global__ void __launch_bounds__(SB)
+argmax_partial_kernel(const float* __restrict__ logits, int vocab, float* __restrict__ part_val,
+                      int* __restrict__ part_idx) {
+    __shared__ ArgMax am_scratch[SB / 64];
+    int b = blockIdx.y, c = blockIdx.x;
+    int per = (vocab + ARGMAX_CHUNKS - 1) / ARGMAX_CHUNKS;
+    int lo = c * per, hi = min(vocab, lo + per);
+    const float* row = logits + (size_t)b * vocab;
+    ArgMax best = {-INFINITY, 0x7fffffff};
+    for (int i = lo + threadIdx.x; i < hi; i += SB) {
+        ArgMax cand = {row[i], i};
+        best = better(best, cand);
+    }
+    best = block_argmax(best, am_scratch);
+    if (threadIdx.x == 0) {
+        part_val[b * ARGMAX_CHUNKS + c] = best.v;
+        part_idx[b * ARGMAX_CHUNKS + c] = best.i;
+    }
+}
+
+__global__ void argmax_final_kernel(const float* __restrict__ part_val, const int* __restrict__ part_idx,
+                                    int* __restrict__ out) {
+    int b = blockIdx.x, lane = threadIdx.x;      // 64 threads
+    ArgMax a = {-INFINITY, 0x7fffffff};
+    if (lane < ARGMAX_CHUNKS) a = ArgMax{part_val[b * ARGMAX_CHUNKS + lane], part_idx[b * ARGMAX_CHUNKS + lane]};
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        ArgMax o;
+        o.v = __shfl_xor(a.v, off, 64);
+        o.i = __shfl_xor(a.i, off, 64);
+        a = better(a, o);
+    }
+    if (lane == 0) out[b] = a.i == 0x7fffffff ? 0 : a.i;
+}
+
+// work: 2 * batch * ARGMAX_CHUNKS 32-bit words of device memory, or null for the one-stage kernel.
+ROCML_EXPORT int rocml_argmax(const float* logits, int batch, int vocab, int* out, void* work,
+                              hipStream_t stream) {
     ROCML_REQUIRE(batch >= 0 && vocab > 0, "argmax: bad sizes B=%d V=%d", batch, vocab);
     if (batch == 0) return 0;
-    argmax_kernel<<<batch, SB, 0, stream>>>(logits, vocab, out);
+    if (work && vocab >= 4096) {
+        float* part_val = (float*)work;
+        int* part_idx = (int*)work + (size_t)batch * ARGMAX_CHUNKS;
+        argmax_partial_kernel<<<dim3(ARGMAX_CHUNKS, batch), SB, 0, stream>>>(logits, vocab, part_val, part_idx);
+        argmax_final_kernel<<<batch, 64, 0, stream>>>(part_val, part_idx, out);
+    } else {
+        argmax_kernel<<<batch, SB, 0, stream>>>(logits, vocab, out);
+    }
     ROCML_CHECK_LAUNCH("argmax");
     return 0;
 }

@@ -45,7 +45,7 @@ _SIGNATURES = {
     },
     "sampling": {
         "rocml_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P],
-        "rocml_argmax": [_P, _I, _I, _P, _P],
+        "rocml_argmax": [_P, _I, _I, _P, _P, _P],
     },
 }
 
@@ -326,12 +326,19 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache
 
 
 # ---- sampling ------------------------------------------------------------------------
-def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
-    _dev(logits, out)
+ARGMAX_WORK_WORDS = 64      # 32-bit words of workspace per row for the two-stage argmax
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor, work: Optional[torch.Tensor] = None) -> None:
+    """First index of each row's maximum.  With ``work`` (``ARGMAX_WORK_WORDS`` 32-bit words
+    per row) long rows are searched by several blocks."""
+    _dev(logits, out, work)
     _want(logits, torch.float32, "logits")
     _want(out, torch.int32, "token output")
     batch, vocab = logits.shape
-    _check("sampling", library("sampling").rocml_argmax(_ptr(logits), batch, vocab, _ptr(out), _stream()))
+    if work is not None and work.numel() * work.element_size() < batch * ARGMAX_WORK_WORDS * 4:
+        raise KernelError("argmax workspace is too small")
+    _check("sampling", library("sampling").rocml_argmax(_ptr(logits), batch, vocab, _ptr(out), _ptr(work), _stream()))
 
 
 def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor,

@@ -38,6 +38,7 @@ class DeviceSampler:
     def __init__(self, device):
         self.device = torch.device(device)
         self._work: Optional[torch.Tensor] = None
+        self._argmax_work: Optional[torch.Tensor] = None
 
     def sample(self, logits: torch.Tensor, seqs: Sequence[SequenceSampling]) -> List[int]:
         """``logits`` is ``[B, V]`` 32-bit on the device, row ``b`` for ``seqs[b]``.  Returns
@@ -46,7 +47,9 @@ class DeviceSampler:
         assert batch == len(seqs)
         out = torch.empty(batch, dtype=torch.int32, device=self.device)
         if all(s.params.is_greedy() and not s.params.penalty_active() for s in seqs):
-            ops.argmax(logits, out)
+            if self._argmax_work is None or self._argmax_work.numel() < batch * ops.ARGMAX_WORK_WORDS:
+                self._argmax_work = torch.empty(max(batch, 64) * ops.ARGMAX_WORK_WORDS, dtype=torch.int32, device=self.device)
+            ops.argmax(logits, out, self._argmax_work)
             return out.cpu().tolist()
         if self._work is None or self._work.numel() < logits.numel():
             self._work = torch.empty(logits.numel(), dtype=torch.float32, device=self.device)

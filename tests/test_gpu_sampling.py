@@ -47,6 +47,14 @@ def test_argmax_takes_the_first_maximum():
     out = torch.empty(5, dtype=torch.int32, device="cuda")
     ops.argmax(logits.cuda(), out)
     assert out.cpu().tolist() == [17, 999, 0, 0, int(logits[4].argmax())]
+    # long rows take the two-stage path: the first maximum still wins, across pieces too
+    long = torch.randn(3, 151936)
+    long[0, 5000] = long[0, 140000] = 50.0
+    long[1, 151935] = 50.0
+    work = torch.empty(3 * ops.ARGMAX_WORK_WORDS, dtype=torch.int32, device="cuda")
+    out = torch.empty(3, dtype=torch.int32, device="cuda")
+    ops.argmax(long.cuda(), out, work)
+    assert out.cpu().tolist() == [5000, 151935, int(long[2].argmax())]
 
 
 def _draw(logits, params_list, us, histories=None):
