@@ -73,42 +73,23 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
 #pragma unroll
     for (int i = 0; i < DT; ++i) o[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    // A piece is 32 keys of one page: its keys (2 x KD loads of 16 bytes per lane) and values
-    // (2 x DT loads of 8 bytes) are all asked for at once, and the next piece of this wave is
-    // asked for before the current one is multiplied, so the memory latency is paid once.
-    uint4 kc[2][KD], kn[2][KD];
-    uint2 vc[2][DT], vn[2][DT];
-    auto load_piece = [&](int piece, uint4 (*kd_)[KD], uint2 (*vd_)[DT]) {
+    for (int piece = wave; piece < n_pieces; piece += 4) {
         int lpage = p_begin + (piece >> 1), half = piece & 1;
         int phys = pages[lpage];
         const bf16_t* kbase = kcache + (((size_t)phys * hkv + kvh) * AM_PAGE + half * 32) * D;
         const bf16_t* vbase = vcache + ((size_t)phys * hkv + kvh) * D * AM_PAGE + half * 32;
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const bf16_t* krow = kbase + (size_t)(u * 16 + col) * D + g * 8;
-#pragma unroll
-            for (int kd = 0; kd < KD; ++kd) kd_[u][kd] = *(const uint4*)(krow + kd * 32);
-        }
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            const bf16_t* vrow = vbase + (size_t)(dt * 16 + col) * AM_PAGE + g * 4;
-            vd_[0][dt] = *(const uint2*)vrow;
-            vd_[1][dt] = *(const uint2*)(vrow + 16);
-        }
-    };
-    if (wave < n_pieces) load_piece(wave, kc, vc);
-    for (int piece = wave; piece < n_pieces; piece += 4) {
-        bool more = piece + 4 < n_pieces;
-        if (more) load_piece(piece + 4, kn, vn);
-        int key0 = (p_begin + (piece >> 1)) * AM_PAGE + (piece & 1) * 32;
+        int key0 = lpage * AM_PAGE + half * 32;
         // scores of 2 x 16 keys: element i of s[u] is key 16u + 4g + i, column = head.
         f32x4_t s[2];
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             s[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            const bf16_t* krow = kbase + (size_t)(u * 16 + col) * D + g * 8;
 #pragma unroll
-            for (int kd = 0; kd < KD; ++kd)
-                s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kc[u][kd]), qf[kd], s[u], 0, 0, 0);
+            for (int kd = 0; kd < KD; ++kd) {
+                bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(krow + kd * 32));
+                s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[kd], s[u], 0, 0, 0);
+            }
         }
         float mx = -INFINITY;
 #pragma unroll
@@ -143,18 +124,11 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         bf16x8_t pf = __builtin_bit_cast(bf16x8_t, pv);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-            bf16x8_t vf = __builtin_bit_cast(bf16x8_t, make_uint4(vc[0][dt].x, vc[0][dt].y, vc[1][dt].x, vc[1][dt].y));
+            const bf16_t* vrow = vbase + (size_t)(dt * 16 + col) * AM_PAGE + g * 4;
+            uint2 a = *(const uint2*)vrow, b = *(const uint2*)(vrow + 16);
+            bf16x8_t vf = __builtin_bit_cast(bf16x8_t, make_uint4(a.x, a.y, b.x, b.y));
             o[dt] = o[dt] * corr;
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[dt], 0, 0, 0);
-        }
-        if (more) {
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-#pragma unroll
-                for (int kd = 0; kd < KD; ++kd) kc[u][kd] = kn[u][kd];
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) vc[u][dt] = vn[u][dt];
-            }
         }
     }
     // merge the four waves in wave order; element i of o[dt] is d = 16 dt + 4g + i, column = head.

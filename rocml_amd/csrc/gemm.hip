@@ -48,13 +48,17 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
         if (allow_lds(gemm_skinny_kernel<MT, EPI, true>, LDS, "gemm")) return 1;
         ready = true;
     }
-    int blocks_n = ceil_div(n, GS_BN);
+    // Wide products without a split get blocks of two waves: more, smaller blocks keep more
+    // loads in flight when nothing else multiplies their number.
+    constexpr bool CAN_NARROW = MT == 1;
+    bool narrow = CAN_NARROW && (EPI == EPI_SWIGLU || n >= 65536);
+    int blocks_n = ceil_div(n, narrow ? 32 : GS_BN);
     int target = MT == 4 ? 256 : 512;
     int splits = target / blocks_n;
     int by_k = k / 512;
     if (splits > by_k) splits = by_k;
     if (splits > 16) splits = 16;
-    if (splits < 1 || EPI == EPI_SWIGLU) splits = 1;     // the gated epilogue needs whole sums
+    if (splits < 1 || EPI == EPI_SWIGLU || narrow) splits = 1;     // the gated epilogue needs whole sums
     long long per_split = (long long)m * n * sizeof(float);
     if (splits > 1 && (long long)splits * per_split > workspace_bytes)
         splits = workspace ? (int)(workspace_bytes / per_split) : 1;
@@ -62,7 +66,11 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
     int k_per_split = round_up(ceil_div(k, splits), GS_KC);
     splits = ceil_div(k, k_per_split);
     dim3 grid(blocks_n, splits);
-    if (splits == 1) {
+    if (splits == 1 && narrow) {
+        if constexpr (CAN_NARROW)
+            gemm_skinny_kernel<MT, EPI, false, 2><<<grid, 128, LDS, stream>>>(
+                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
+    } else if (splits == 1) {
         gemm_skinny_kernel<MT, EPI, false><<<grid, GS_THREADS, LDS, stream>>>(
             (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
     } else {

@@ -24,7 +24,12 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;   // 16 bytes as a native vector: a
+// conditional between two of these is a register select, between two uint4 structs it goes
+// through memory and drags whole arrays into scratch
+
 __device__ __forceinline__ bf16x8_t as_frag(uint4 v) { return __builtin_bit_cast(bf16x8_t, v); }
+__device__ __forceinline__ bf16x8_t as_frag4(u32x4_t v) { return __builtin_bit_cast(bf16x8_t, v); }
 
 // Unconditional 16-byte load from an address the caller has clamped into range, zeroed
 // afterwards when the element is outside the matrix: a load under a branch would be waited for
@@ -51,15 +56,15 @@ __device__ __forceinline__ void epilogue_store(void* out, size_t idx, float v) {
 
 // ---- many rows ---------------------------------------------------------------------------
 constexpr int GM_BM = 128, GM_BN = 128, GM_BK = 64, GM_THREADS = 256;
-constexpr int GM_ROW = GM_BK / 8 + 1;                 // uint4 per LDS row, one of padding
-constexpr int GM_TILE = GM_BM * GM_ROW;               // uint4 per operand tile
+constexpr int GM_ROW = GM_BK / 8 + 1;                 // u32x4_t per LDS row, one of padding
+constexpr int GM_TILE = GM_BM * GM_ROW;               // u32x4_t per operand tile
 constexpr int GM_LDS_BYTES = 2 * 2 * GM_TILE * 16;    // two stages, two operands
 
 template <int EPI>
 __global__ void __launch_bounds__(GM_THREADS)
 gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw,
                  void* __restrict__ out, int ldo, int m, int n, int k, int tiles_m, int n_tiles) {
-    extern __shared__ uint4 gm_smem[];
+    extern __shared__ u32x4_t gm_smem[];
     int per_xcd = gridDim.x / 8;
     int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
     if (logical >= n_tiles) return;
@@ -68,7 +73,11 @@ gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
     int wm = wave >> 1, wn = wave & 1;
     int lrow = tid >> 3, lkc = tid & 7;
     int nk = (k + GM_BK - 1) / GM_BK;
-    uint4 ra[4], rb[4];
+    // The global loads of the next K stage are issued before the current stage is multiplied
+    // and written to the other LDS buffer afterwards: one barrier per stage.  (Loading two
+    // stages ahead was tried: the compiler then keeps two sets of accumulators and the kernel
+    // is slower.)
+    u32x4_t ra[4], rb[4];
     f32x16_t acc[2][2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -77,46 +86,51 @@ gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    auto load_global = [&](int kt) {
-        int gk = kt * GM_BK + lkc * 8;
-        bool kin = gk < k;
+    // Loads go to clamped addresses and are used as they come: rows beyond M or N only feed
+    // outputs that are never stored.  Only a 16-byte piece beyond K must count as zero, and that
+    // is decided when the piece is written to LDS, long after the load was issued (a select
+    // right behind the load would make the wave wait for it there).
+    const bf16_t* xrow[4];
+    const bf16_t* wrow[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            int row = lrow + 32 * i;
-            bool oka = kin && (m0 + row) < m;
-            bool okb = kin && (n0 + row) < n;
-            ra[i] = load16_or_zero(x + (size_t)min(m0 + row, m - 1) * ldx + (kin ? gk : 0), oka);
-            rb[i] = load16_or_zero(w + (size_t)min(n0 + row, n - 1) * ldw + (kin ? gk : 0), okb);
-        }
-    };
-    auto store_lds = [&](int buf) {
-        uint4* sa = gm_smem + buf * 2 * GM_TILE;
-        uint4* sb = sa + GM_TILE;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            int row = lrow + 32 * i;
-            sa[row * GM_ROW + lkc] = ra[i];
-            sb[row * GM_ROW + lkc] = rb[i];
-        }
-    };
-
-    load_global(0);
-    store_lds(0);
-    __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-        int buf = kt & 1;
-        bool more = kt + 1 < nk;
-        if (more) load_global(kt + 1);
-        const uint4* sa = gm_smem + buf * 2 * GM_TILE;
-        const uint4* sb = sa + GM_TILE;
+    for (int i = 0; i < 4; ++i) {
+        xrow[i] = x + (size_t)min(m0 + lrow + 32 * i, m - 1) * ldx;
+        wrow[i] = w + (size_t)min(n0 + lrow + 32 * i, n - 1) * ldw;
+    }
+    // Written as macros over the register arrays: handed to a function through a pointer, the
+    // arrays would be kept in scratch memory and every load waited for at once.
+#define GM_LOAD_GLOBAL(kt_)                                                  \
+    {                                                                        \
+        int gk_ = (kt_) * GM_BK + lkc * 8;                                   \
+        gk_ = gk_ < k ? gk_ : 0;                                             \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i) {                      \
+            ra[i] = *(const u32x4_t*)(xrow[i] + gk_);                        \
+            rb[i] = *(const u32x4_t*)(wrow[i] + gk_);                        \
+        }                                                                    \
+    }
+#define GM_STORE_LDS(kt_, buf_)                                              \
+    {                                                                        \
+        u32x4_t* sa_ = gm_smem + (buf_) * 2 * GM_TILE;                         \
+        u32x4_t* sb_ = sa_ + GM_TILE;                                          \
+        bool kin_ = (kt_) * GM_BK + lkc * 8 < k;                             \
+        const u32x4_t zero_ = {0u, 0u, 0u, 0u};                          \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i) {                      \
+            int row_ = lrow + 32 * i;                                        \
+            sa_[row_ * GM_ROW + lkc] = kin_ ? ra[i] : zero_;                 \
+            sb_[row_ * GM_ROW + lkc] = kin_ ? rb[i] : zero_;                 \
+        }                                                                    \
+    }
+    auto multiply = [&](int buf) {
+        const u32x4_t* sa = gm_smem + buf * 2 * GM_TILE;
+        const u32x4_t* sb = sa + GM_TILE;
 #pragma unroll
         for (int kk = 0; kk < GM_BK / 16; ++kk) {
             bf16x8_t a[2], b[2];
             int col = kk * 2 + (lane >> 5);
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
-                a[i] = as_frag(sa[(wm * 64 + i * 32 + (lane & 31)) * GM_ROW + col]);
-                b[i] = as_frag(sb[(wn * 64 + i * 32 + (lane & 31)) * GM_ROW + col]);
+                a[i] = as_frag4(sa[(wm * 64 + i * 32 + (lane & 31)) * GM_ROW + col]);
+                b[i] = as_frag4(sb[(wn * 64 + i * 32 + (lane & 31)) * GM_ROW + col]);
             }
 #pragma unroll
             for (int i = 0; i < 2; ++i)
@@ -124,9 +138,21 @@ gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
                 for (int j = 0; j < 2; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
         }
-        if (more) store_lds(buf ^ 1);
+    };
+
+    GM_LOAD_GLOBAL(0)
+    GM_STORE_LDS(0, 0)
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+        int buf = kt & 1;
+        bool more = kt + 1 < nk;
+        if (more) GM_LOAD_GLOBAL(kt + 1)
+        multiply(buf);
+        if (more) GM_STORE_LDS(kt + 1, buf ^ 1)
         __syncthreads();
     }
+#undef GM_LOAD_GLOBAL
+#undef GM_STORE_LDS
     // Accumulator element e of a lane: row 8*(e/4) + 4*(lane/32) + e%4, column lane%32.
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -153,22 +179,27 @@ constexpr int GS_BN = 64, GS_KC = 256, GS_THREADS = 256;
 constexpr int GS_ROW = GS_KC / 8 + 1;                 // uint4 per LDS row of activations
 
 // PARTIAL: write 32-bit partial sums [split][M][N] instead of the epilogue.
-template <int MT, int EPI, bool PARTIAL>
-__global__ void __launch_bounds__(GS_THREADS)
+// Loads are never followed by a select: addresses beyond the matrix are clamped to a place
+// inside it, rows beyond M or N only feed outputs that are not stored, and a piece beyond K is
+// zeroed on the activation side when it is written to LDS (the weight beside it is then some
+// finite weight times zero).  A select right behind a load would make the wave wait for the
+// load there and undo the overlap of the next chunk's loads with this chunk's products.
+template <int MT, int EPI, bool PARTIAL, int WAVES = 4>
+__global__ void __launch_bounds__(64 * WAVES)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw,
                    void* __restrict__ out, int ldo, int m, int n, int k, int k_per_split) {
-    extern __shared__ uint4 gs_smem[];                // [2][MT*16][GS_ROW]
+    extern __shared__ u32x4_t gs_smem[];              // [2][MT*16][GS_ROW]
     constexpr int ROWS = MT * 16;
-    constexpr int XCHUNKS = ROWS * (GS_KC / 8) / GS_THREADS;   // 16-byte pieces per thread
+    constexpr int THREADS = 64 * WAVES;
+    constexpr int XCHUNKS = ROWS * (GS_KC / 8) / THREADS;   // 16-byte pieces per thread
     int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    int n0 = blockIdx.x * GS_BN + wave * 16;
+    int n0 = blockIdx.x * (16 * WAVES) + wave * 16;
     int ks = blockIdx.y * k_per_split;
     int ke = min(k, ks + k_per_split);
     int n_chunks = (ke - ks + GS_KC - 1) / GS_KC;
-    int wrow = n0 + (lane & 15);
-    bool wok = wrow < n;
-    const bf16_t* wbase = w + (size_t)(wok ? wrow : 0) * ldw + (lane >> 4) * 8;
-    uint4 wcur[8], wnext[8], xr[XCHUNKS];
+    const bf16_t* wsafe = w + (size_t)min(n0 + (lane & 15), n - 1) * ldw;
+    const bf16_t* wbase = wsafe + (lane >> 4) * 8;
+    u32x4_t wcur[8], wnext[8], xr[XCHUNKS];
     f32x4_t acc[MT];
 #pragma unroll
     for (int i = 0; i < MT; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -177,68 +208,68 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restri
     // power of two, and blocks that all read the same K window at once would queue up on a few
     // memory channels.
     int rot = (blockIdx.x * 5 + blockIdx.y * 3) % n_chunks;
-    auto chunk_base = [&](int c) {
-        int cc = c + rot;
-        if (cc >= n_chunks) cc -= n_chunks;
-        return ks + cc * GS_KC;
-    };
-    auto load_w = [&](int c, uint4* dst) {
-        int kb = chunk_base(c);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            int gk = kb + j * 32 + (lane >> 4) * 8;
-            bool ok = gk < ke;
-            dst[j] = load16_or_zero(ok ? wbase + kb + j * 32 : w, wok && ok);
-        }
-    };
-    auto load_x = [&](int c) {
-        int kb = chunk_base(c);
-#pragma unroll
-        for (int i = 0; i < XCHUNKS; ++i) {
-            int piece = tid + i * GS_THREADS;
-            int row = piece / (GS_KC / 8), kc = piece % (GS_KC / 8);
-            int gk = kb + kc * 8;
-            bool ok = gk < ke;
-            xr[i] = load16_or_zero(ok ? x + (size_t)min(row, m - 1) * ldx + gk : x, ok && row < m);
-        }
-    };
-    auto store_x = [&](int buf) {
-        uint4* sx = gs_smem + buf * ROWS * GS_ROW;
-#pragma unroll
-        for (int i = 0; i < XCHUNKS; ++i) {
-            int piece = tid + i * GS_THREADS;
-            sx[(piece / (GS_KC / 8)) * GS_ROW + piece % (GS_KC / 8)] = xr[i];
-        }
-    };
+#define GS_CHUNK_BASE(c_) (ks + (((c_) + rot) >= n_chunks ? (c_) + rot - n_chunks : (c_) + rot) * GS_KC)
+#define GS_LOAD_W(c_, dst_)                                                                     \
+    {                                                                                           \
+        int kb_ = GS_CHUNK_BASE(c_);                                                            \
+        _Pragma("unroll") for (int j = 0; j < 8; ++j) {                                         \
+            bool in_ = kb_ + j * 32 + (lane >> 4) * 8 < ke;                                     \
+            dst_[j] = *(const u32x4_t*)(in_ ? wbase + kb_ + j * 32 : wsafe);                    \
+        }                                                                                       \
+    }
+#define GS_LOAD_X(c_)                                                                           \
+    {                                                                                           \
+        int kb_ = GS_CHUNK_BASE(c_);                                                            \
+        _Pragma("unroll") for (int i = 0; i < XCHUNKS; ++i) {                                   \
+            int piece_ = tid + i * THREADS;                                                  \
+            int row_ = piece_ / (GS_KC / 8), gk_ = kb_ + (piece_ % (GS_KC / 8)) * 8;            \
+            xr[i] = *(const u32x4_t*)(gk_ < ke ? x + (size_t)min(row_, m - 1) * ldx + gk_ : x); \
+        }                                                                                       \
+    }
+#define GS_STORE_X(c_, buf_)                                                                    \
+    {                                                                                           \
+        int kb_ = GS_CHUNK_BASE(c_);                                                            \
+        u32x4_t* sx_ = gs_smem + (buf_) * ROWS * GS_ROW;                                        \
+        const u32x4_t zero_ = {0u, 0u, 0u, 0u};                                                 \
+        _Pragma("unroll") for (int i = 0; i < XCHUNKS; ++i) {                                   \
+            int piece_ = tid + i * THREADS;                                                  \
+            int kc_ = piece_ % (GS_KC / 8);                                                     \
+            sx_[(piece_ / (GS_KC / 8)) * GS_ROW + kc_] = kb_ + kc_ * 8 < ke ? xr[i] : zero_;    \
+        }                                                                                       \
+    }
 
-    load_w(0, wcur);
-    load_x(0);
-    store_x(0);
+    GS_LOAD_W(0, wcur)
+    GS_LOAD_X(0)
+    GS_STORE_X(0, 0)
     __syncthreads();
     for (int c = 0; c < n_chunks; ++c) {
         int buf = c & 1;
         bool more = c + 1 < n_chunks;
         if (more) {
-            load_w(c + 1, wnext);
-            load_x(c + 1);
+            GS_LOAD_W(c + 1, wnext)
+            GS_LOAD_X(c + 1)
         }
-        const uint4* sx = gs_smem + buf * ROWS * GS_ROW;
+        const u32x4_t* sx = gs_smem + buf * ROWS * GS_ROW;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            bf16x8_t a = as_frag(wcur[j]);
+            bf16x8_t a = as_frag4(wcur[j]);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-                bf16x8_t b = as_frag(sx[(mt * 16 + (lane & 15)) * GS_ROW + j * 4 + (lane >> 4)]);
+                bf16x8_t b = as_frag4(sx[(mt * 16 + (lane & 15)) * GS_ROW + j * 4 + (lane >> 4)]);
                 acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
             }
         }
         if (more) {
-            store_x(buf ^ 1);
+            GS_STORE_X(c + 1, buf ^ 1)
 #pragma unroll
             for (int j = 0; j < 8; ++j) wcur[j] = wnext[j];
         }
         __syncthreads();
     }
+#undef GS_CHUNK_BASE
+#undef GS_LOAD_W
+#undef GS_LOAD_X
+#undef GS_STORE_X
     // Accumulator element e of a lane: weight row (lane/16)*4 + e, activation row lane%16.
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -285,28 +316,31 @@ gemm_kpar_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
     int bs = split * k_per_split, be = min(k, bs + k_per_split);
     int quarter = (((be - bs + 3) / 4) + 31) / 32 * 32;
     int ks = min(be, bs + wave * quarter), ke = min(be, ks + quarter);
-    int wrow = tile * 16 + col;
-    bool wok = wrow < n, xok = col < m;
-    const bf16_t* wp = w + (size_t)(wok ? wrow : 0) * ldw + g * 8;
-    const bf16_t* xp = x + (size_t)(xok ? col : 0) * ldx + g * 8;
-    uint4 wc[8], xc[8], wn[8], xn[8];
+    bool xok = col < m;
+    const bf16_t* wsafe = w + (size_t)min(tile * 16 + col, n - 1) * ldw;
+    const bf16_t* xsafe = x + (size_t)min(col, m - 1) * ldx;
+    const bf16_t* wp = wsafe + g * 8;
+    const bf16_t* xp = xsafe + g * 8;
+    u32x4_t wc[8], xc[8], wn[8], xn[8];
     f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    auto load = [&](int kb, uint4* wd, uint4* xd) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            int gk = kb + j * 32;
-            bool ok = gk + g * 8 < ke;
-            wd[j] = load16_or_zero(ok ? wp + gk : w, ok && wok);
-            xd[j] = load16_or_zero(ok ? xp + gk : x, ok && xok);
-        }
-    };
-    if (ks < ke) load(ks, wc, xc);
+    // No select behind a load (see the few-rows kernel): clamped addresses, and the activations
+    // of a piece beyond K are zeroed just before they are multiplied.
+#define GK_LOAD(kb_, wd_, xd_)                                                \
+    _Pragma("unroll") for (int j = 0; j < 8; ++j) {                           \
+        bool in_ = (kb_) + j * 32 + g * 8 < ke;                               \
+        wd_[j] = *(const u32x4_t*)(in_ ? wp + (kb_) + j * 32 : wsafe);        \
+        xd_[j] = *(const u32x4_t*)(in_ ? xp + (kb_) + j * 32 : xsafe);        \
+    }
+    if (ks < ke) GK_LOAD(ks, wc, xc)
     for (int kb = ks; kb < ke; kb += GK_KC) {
         bool more = kb + GK_KC < ke;
-        if (more) load(kb + GK_KC, wn, xn);
+        if (more) GK_LOAD(kb + GK_KC, wn, xn)
+        const u32x4_t zero = {0u, 0u, 0u, 0u};
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(wc[j]), as_frag(xc[j]), acc, 0, 0, 0);
+        for (int j = 0; j < 8; ++j) {
+            u32x4_t xv = kb + j * 32 + g * 8 < ke ? xc[j] : zero;
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag4(wc[j]), as_frag4(xv), acc, 0, 0, 0);
+        }
         if (more) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
@@ -315,6 +349,7 @@ gemm_kpar_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
             }
         }
     }
+#undef GK_LOAD
 #pragma unroll
     for (int e = 0; e < 4; ++e) red[wave][lane][e] = acc[e];
     __syncthreads();

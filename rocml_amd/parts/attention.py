@@ -70,7 +70,7 @@ class Attention(Mixer):
         if step.max_new != 1:
             return 0
         blocks = step.n_tokens * self.spec.n_kv_heads
-        return max(1, min(1024 // blocks, cache.block_table.shape[1], 64))
+        return max(1, min(512 // blocks, cache.block_table.shape[1], 64))
 
     def forward(self, step, xn, x_accum, cache, owns_cache: bool) -> None:
         s = self.spec
