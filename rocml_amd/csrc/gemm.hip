@@ -8,7 +8,8 @@
 
 ROCML_LAST_ERROR_FN(gemm)
 
-enum GemmAlgo : int { ALGO_AUTO = 0, ALGO_PLAIN = 1, ALGO_MFMA_TILE = 2, ALGO_MFMA_SKINNY = 3, ALGO_MFMA_KPAR = 4 };
+enum GemmAlgo : int { ALGO_AUTO = 0, ALGO_PLAIN = 1, ALGO_MFMA_TILE = 2, ALGO_MFMA_SKINNY = 3, ALGO_MFMA_KPAR = 4,
+                      ALGO_MFMA_TILE256 = 5 };
 
 static int round_up(int a, int b) { return (a + b - 1) / b * b; }
 
@@ -20,20 +21,35 @@ static int allow_lds(K kernel, int bytes, const char* name) {
     return 0;
 }
 
-template <int EPI>
-static int launch_mfma_tile(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m,
-                            int n, int k, hipStream_t stream) {
+template <int EPI, typename T>
+static int launch_mfma_tile_as(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m,
+                               int n, int k, hipStream_t stream) {
     static bool ready = false;
     if (!ready) {
-        if (allow_lds(gemm_mfma_kernel<EPI>, GM_LDS_BYTES, "gemm")) return 1;
+        if (allow_lds(gemm_mfma_kernel<EPI, T>, T::LDS_BYTES, "gemm")) return 1;
         ready = true;
     }
-    int tiles_m = ceil_div(m, GM_BM), tiles_n = ceil_div(n, GM_BN);
+    int tiles_m = ceil_div(m, T::BM), tiles_n = ceil_div(n, T::BN);
     int n_tiles = tiles_m * tiles_n;
     int grid = round_up(n_tiles, 8);
-    gemm_mfma_kernel<EPI><<<grid, GM_THREADS, GM_LDS_BYTES, stream>>>(
+    gemm_mfma_kernel<EPI, T><<<grid, T::THREADS, T::LDS_BYTES, stream>>>(
         (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, tiles_m, n_tiles);
     return 0;
+}
+
+// big: 0 = choose, 1 = 128x128 tiles, 2 = 256x256 tiles.  Measured on large products the big
+// tile reaches about 975 TFLOP/s and the small one about 800, but a CU holds one big tile or
+// two small ones at a time, and the last round of tiles may leave CUs idle: the choice weighs
+// the speed with the share of the 256 CUs that the rounds keep busy.
+template <int EPI>
+static int launch_mfma_tile(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m,
+                            int n, int k, int big, hipStream_t stream) {
+    double t256 = (double)ceil_div(m, 256) * ceil_div(n, 256), t128 = (double)ceil_div(m, 128) * ceil_div(n, 128);
+    double score256 = 975.0 * t256 / (ceil_div((long long)t256, 256) * 256.0);
+    double score128 = 800.0 * t128 / (ceil_div((long long)t128, 512) * 512.0);
+    bool use256 = big == 2 || (big == 0 && score256 > score128);
+    if (use256) return launch_mfma_tile_as<EPI, GemmTile256>(x, ldx, w, ldw, out, ldo, m, n, k, stream);
+    return launch_mfma_tile_as<EPI, GemmTile128>(x, ldx, w, ldw, out, ldo, m, n, k, stream);
 }
 
 struct SplitPlan { int defer; int* deferred; };
@@ -159,7 +175,7 @@ ROCML_EXPORT int rocml_splitk_reduce(const float* partials, void* out, int out_d
 }
 
 // algo: 0 = choose, 1 = plain tiled kernel, 2 = MFMA tile kernel, 3 = MFMA few-rows kernel (M <= 64),
-// 4 = MFMA kernel for at most 16 rows.
+// 4 = MFMA kernel for at most 16 rows, 5 = MFMA tile kernel with 256x256 tiles.
 // accumulate: out += product (out must be 32-bit); this is the residual sum's epilogue.
 // epilogue: 0 = none; 1 = gated activation: W's rows are (gate_j, up_j) pairs and out is
 //   [M, N/2] = silu(gate) * up.
@@ -180,7 +196,7 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
     ROCML_REQUIRE(ldx >= k && ldw >= k && ldo >= out_cols, "gemm: row strides (%d, %d, %d) below (K, K, N)",
                   ldx, ldw, ldo);
     ROCML_REQUIRE(!accumulate || out_dtype == ROCML_F32, "gemm: accumulation needs a 32-bit output");
-    ROCML_REQUIRE(algo >= ALGO_AUTO && algo <= ALGO_MFMA_KPAR, "gemm: unknown algorithm %d", algo);
+    ROCML_REQUIRE(algo >= ALGO_AUTO && algo <= ALGO_MFMA_TILE256, "gemm: unknown algorithm %d", algo);
     ROCML_REQUIRE(!defer || deferred_splits, "gemm: deferring needs a place to report the splits");
     if (m == 0) return 0;
     bool bf16_in = x_dtype == ROCML_BF16 && w_dtype == ROCML_BF16;
@@ -207,7 +223,8 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
         bool kpar = algo == ALGO_MFMA_KPAR || (algo == ALGO_AUTO && m <= 2);   // beyond two rows the activations read from L2 cost more than the block sharing of the few-rows kernel
         if (kpar) rc = BY_EPI(launch_kpar, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
         else if (skinny) rc = BY_EPI(launch_skinny_m, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
-        else rc = BY_EPI(launch_mfma_tile, x, ldx, w, ldw, out, ldo, m, n, k, stream);
+        else rc = BY_EPI(launch_mfma_tile, x, ldx, w, ldw, out, ldo, m, n, k,
+                         algo == ALGO_MFMA_TILE ? 1 : algo == ALGO_MFMA_TILE256 ? 2 : 0, stream);
 #undef BY_EPI
         if (rc) return rc;
         ROCML_CHECK_LAUNCH("gemm");

@@ -55,34 +55,49 @@ __device__ __forceinline__ void epilogue_store(void* out, size_t idx, float v) {
 }
 
 // ---- many rows ---------------------------------------------------------------------------
-constexpr int GM_BM = 128, GM_BN = 128, GM_BK = 64, GM_THREADS = 256;
+// One kernel, two shapes (see GemmTile below): 128x128 with four waves for most products, and
+// 256x256 with eight waves (two per SIMD, each 128x64) for products wide enough to give every
+// CU several such tiles: four times the products per LDS byte and per barrier.
+constexpr int GM_BK = 64;
 constexpr int GM_ROW = GM_BK / 8 + 1;                 // u32x4_t per LDS row, one of padding
-constexpr int GM_TILE = GM_BM * GM_ROW;               // u32x4_t per operand tile
-constexpr int GM_LDS_BYTES = 2 * 2 * GM_TILE * 16;    // two stages, two operands
 
-template <int EPI>
-__global__ void __launch_bounds__(GM_THREADS)
+template <int WAVES_M_, int WAVES_N_, int TM_, int TN_>
+struct GemmTile {
+    static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;   // waves along M and N
+    static constexpr int TM = TM_, TN = TN_;                        // 32x32 MFMA tiles per wave
+    static constexpr int BM = WAVES_M * TM * 32, BN = WAVES_N * TN * 32;
+    static constexpr int THREADS = 64 * WAVES_M * WAVES_N;
+    static constexpr int PASS_ROWS = THREADS / 8;                   // tile rows one pass loads
+    static constexpr int PA = BM / PASS_ROWS, PB = BN / PASS_ROWS;  // passes per operand
+    static constexpr int LDS_BYTES = 2 * (BM + BN) * GM_ROW * 16;   // two stages
+};
+using GemmTile128 = GemmTile<2, 2, 2, 2>;
+using GemmTile256 = GemmTile<2, 4, 4, 2>;
+
+template <int EPI, typename T>
+__global__ void __launch_bounds__(T::THREADS)
 gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw,
                  void* __restrict__ out, int ldo, int m, int n, int k, int tiles_m, int n_tiles) {
-    extern __shared__ u32x4_t gm_smem[];
+    extern __shared__ u32x4_t gm_smem[];              // [2 stages][A: BM rows | B: BN rows][GM_ROW]
+    constexpr int STAGE = (T::BM + T::BN) * GM_ROW;
     int per_xcd = gridDim.x / 8;
     int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
     if (logical >= n_tiles) return;
-    int m0 = (logical % tiles_m) * GM_BM, n0 = (logical / tiles_m) * GM_BN;
+    int m0 = (logical % tiles_m) * T::BM, n0 = (logical / tiles_m) * T::BN;
     int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    int wm = wave >> 1, wn = wave & 1;
+    int wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;
     int lrow = tid >> 3, lkc = tid & 7;
     int nk = (k + GM_BK - 1) / GM_BK;
     // The global loads of the next K stage are issued before the current stage is multiplied
     // and written to the other LDS buffer afterwards: one barrier per stage.  (Loading two
     // stages ahead was tried: the compiler then keeps two sets of accumulators and the kernel
     // is slower.)
-    u32x4_t ra[4], rb[4];
-    f32x16_t acc[2][2];
+    u32x4_t ra[T::PA], rb[T::PB];
+    f32x16_t acc[T::TM][T::TN];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < T::TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < T::TN; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
@@ -90,52 +105,49 @@ gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
     // outputs that are never stored.  Only a 16-byte piece beyond K must count as zero, and that
     // is decided when the piece is written to LDS, long after the load was issued (a select
     // right behind the load would make the wave wait for it there).
-    const bf16_t* xrow[4];
-    const bf16_t* wrow[4];
+    const bf16_t* xrow[T::PA];
+    const bf16_t* wrow[T::PB];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        xrow[i] = x + (size_t)min(m0 + lrow + 32 * i, m - 1) * ldx;
-        wrow[i] = w + (size_t)min(n0 + lrow + 32 * i, n - 1) * ldw;
-    }
+    for (int i = 0; i < T::PA; ++i) xrow[i] = x + (size_t)min(m0 + lrow + T::PASS_ROWS * i, m - 1) * ldx;
+#pragma unroll
+    for (int i = 0; i < T::PB; ++i) wrow[i] = w + (size_t)min(n0 + lrow + T::PASS_ROWS * i, n - 1) * ldw;
     // Written as macros over the register arrays: handed to a function through a pointer, the
     // arrays would be kept in scratch memory and every load waited for at once.
-#define GM_LOAD_GLOBAL(kt_)                                                  \
-    {                                                                        \
-        int gk_ = (kt_) * GM_BK + lkc * 8;                                   \
-        gk_ = gk_ < k ? gk_ : 0;                                             \
-        _Pragma("unroll") for (int i = 0; i < 4; ++i) {                      \
-            ra[i] = *(const u32x4_t*)(xrow[i] + gk_);                        \
-            rb[i] = *(const u32x4_t*)(wrow[i] + gk_);                        \
-        }                                                                    \
+#define GM_LOAD_GLOBAL(kt_)                                                                      \
+    {                                                                                            \
+        int gk_ = (kt_) * GM_BK + lkc * 8;                                                       \
+        gk_ = gk_ < k ? gk_ : 0;                                                                 \
+        _Pragma("unroll") for (int i = 0; i < T::PA; ++i) ra[i] = *(const u32x4_t*)(xrow[i] + gk_); \
+        _Pragma("unroll") for (int i = 0; i < T::PB; ++i) rb[i] = *(const u32x4_t*)(wrow[i] + gk_); \
     }
-#define GM_STORE_LDS(kt_, buf_)                                              \
-    {                                                                        \
-        u32x4_t* sa_ = gm_smem + (buf_) * 2 * GM_TILE;                         \
-        u32x4_t* sb_ = sa_ + GM_TILE;                                          \
-        bool kin_ = (kt_) * GM_BK + lkc * 8 < k;                             \
-        const u32x4_t zero_ = {0u, 0u, 0u, 0u};                          \
-        _Pragma("unroll") for (int i = 0; i < 4; ++i) {                      \
-            int row_ = lrow + 32 * i;                                        \
-            sa_[row_ * GM_ROW + lkc] = kin_ ? ra[i] : zero_;                 \
-            sb_[row_ * GM_ROW + lkc] = kin_ ? rb[i] : zero_;                 \
-        }                                                                    \
+#define GM_STORE_LDS(kt_, buf_)                                                                  \
+    {                                                                                            \
+        u32x4_t* sa_ = gm_smem + (buf_) * STAGE;                                                 \
+        u32x4_t* sb_ = sa_ + T::BM * GM_ROW;                                                     \
+        bool kin_ = (kt_) * GM_BK + lkc * 8 < k;                                                 \
+        const u32x4_t zero_ = {0u, 0u, 0u, 0u};                                                  \
+        _Pragma("unroll") for (int i = 0; i < T::PA; ++i)                                        \
+            sa_[(lrow + T::PASS_ROWS * i) * GM_ROW + lkc] = kin_ ? ra[i] : zero_;                \
+        _Pragma("unroll") for (int i = 0; i < T::PB; ++i)                                        \
+            sb_[(lrow + T::PASS_ROWS * i) * GM_ROW + lkc] = kin_ ? rb[i] : zero_;                \
     }
     auto multiply = [&](int buf) {
-        const u32x4_t* sa = gm_smem + buf * 2 * GM_TILE;
-        const u32x4_t* sb = sa + GM_TILE;
+        const u32x4_t* sa = gm_smem + buf * STAGE;
+        const u32x4_t* sb = sa + T::BM * GM_ROW;
 #pragma unroll
         for (int kk = 0; kk < GM_BK / 16; ++kk) {
-            bf16x8_t a[2], b[2];
+            bf16x8_t a[T::TM], b[T::TN];
             int col = kk * 2 + (lane >> 5);
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                a[i] = as_frag4(sa[(wm * 64 + i * 32 + (lane & 31)) * GM_ROW + col]);
-                b[i] = as_frag4(sb[(wn * 64 + i * 32 + (lane & 31)) * GM_ROW + col]);
-            }
+            for (int i = 0; i < T::TM; ++i)
+                a[i] = as_frag4(sa[(wm * T::TM * 32 + i * 32 + (lane & 31)) * GM_ROW + col]);
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int j = 0; j < T::TN; ++j)
+                b[j] = as_frag4(sb[(wn * T::TN * 32 + j * 32 + (lane & 31)) * GM_ROW + col]);
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+            for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+                for (int j = 0; j < T::TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
         }
     };
@@ -155,13 +167,13 @@ gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
 #undef GM_STORE_LDS
     // Accumulator element e of a lane: row 8*(e/4) + 4*(lane/32) + e%4, column lane%32.
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < T::TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            int gn = n0 + wn * 64 + j * 32 + (lane & 31);
+        for (int j = 0; j < T::TN; ++j) {
+            int gn = n0 + (wn * T::TN + j) * 32 + (lane & 31);
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                int gm = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                int gm = m0 + (wm * T::TM + i) * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
                 if (EPI == EPI_SWIGLU) {
                     // neighbouring lanes hold neighbouring columns: the even one has the gate
                     float other = __shfl_xor(acc[i][j][e], 1, 64);
