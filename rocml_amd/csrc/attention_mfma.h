@@ -214,7 +214,7 @@ struct PrefillLds {
 };
 
 template <int D>
-__global__ void __launch_bounds__(AM_THREADS)
+__global__ void __launch_bounds__(AM_THREADS, D <= 128 ? 2 : 1)
 attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                          const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
                          const int* __restrict__ block_table, int bt_width,
@@ -230,8 +230,9 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     int h2 = lane >> 5, col = lane & 31;
     int h = blockIdx.y, kvh = h / (hq / hkv);
-    // which sequence and which of its query tiles
-    int tile = blockIdx.x, b = 0, tok0 = 0, n_new = 0;
+    // which sequence and which of its query tiles; the last tile of a sequence sees the most
+    // keys, so tiles are handed out from the back: long blocks start first
+    int tile = gridDim.x - 1 - blockIdx.x, b = 0, tok0 = 0, n_new = 0;
     for (; b < n_seqs; ++b) {
         tok0 = cu_seqlens[b];
         n_new = cu_seqlens[b + 1] - tok0;
@@ -272,28 +273,44 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
 #pragma unroll
         for (int e = 0; e < 16; ++e) o[i][e] = 0.f;
 
-    for (int lpage = blk_first_key / AM_PAGE; lpage <= blk_last_key / AM_PAGE; ++lpage) {
-        int phys = pages[lpage];
-        const uint4* gk = (const uint4*)(kcache + ((size_t)phys * hkv + kvh) * AM_PAGE * D);
-        const uint4* gv = (const uint4*)(vcache + ((size_t)phys * hkv + kvh) * D * AM_PAGE);
+    // A page's keys and values wait in registers while the page before it is multiplied out of
+    // LDS: the loads of page p + 1 are issued right after page p has been written to LDS.
+    typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+    constexpr int K_PIECES = AM_PAGE * D / 8 / AM_THREADS, V_PIECES = D * AM_PAGE / 8 / AM_THREADS;
+    u32x4 kreg[K_PIECES], vreg[V_PIECES];
+    int first_page = blk_first_key / AM_PAGE, last_page = blk_last_key / AM_PAGE;
+#define AM_LOAD_PAGE(lp_)                                                                         \
+    {                                                                                             \
+        int phys_ = pages[lp_];                                                                   \
+        const u32x4* gk_ = (const u32x4*)(kcache + ((size_t)phys_ * hkv + kvh) * AM_PAGE * D);    \
+        const u32x4* gv_ = (const u32x4*)(vcache + ((size_t)phys_ * hkv + kvh) * D * AM_PAGE);    \
+        _Pragma("unroll") for (int i = 0; i < K_PIECES; ++i) kreg[i] = gk_[tid + i * AM_THREADS]; \
+        _Pragma("unroll") for (int i = 0; i < V_PIECES; ++i) vreg[i] = gv_[tid + i * AM_THREADS]; \
+    }
+    // the wave's rows see every key of a 32-key piece when the piece lies at or below the first
+    // row's position and at or above the last row's window start; only then masking is skipped
+    int wave_min_pos = pos0 + w_lo;
+    int wave_max_lo = window > 0 ? max(0, pos0 + w_hi - window + 1) : 0;
+    bool wave_full = w_hi - w_lo == 31;
+    AM_LOAD_PAGE(first_page)
+    for (int lpage = first_page; lpage <= last_page; ++lpage) {
         __syncthreads();                                // the previous page has been consumed
-        constexpr int K_PIECES = AM_PAGE * D / 8, V_PIECES = D * AM_PAGE / 8;
 #pragma unroll
-        for (int i = 0; i < K_PIECES / AM_THREADS; ++i) {
+        for (int i = 0; i < K_PIECES; ++i) {
             int piece = tid + i * AM_THREADS;
             int key = piece / (D / 8), dc = piece % (D / 8);
-            *(uint4*)(sk + key * L::K_ROW + dc * 8) = gk[piece];
+            *(u32x4*)(sk + key * L::K_ROW + dc * 8) = kreg[i];
         }
 #pragma unroll
-        for (int i = 0; i < V_PIECES / AM_THREADS; ++i) {
+        for (int i = 0; i < V_PIECES; ++i) {
             int piece = tid + i * AM_THREADS;
             int d = piece / 8, kc = piece % 8;
-            uint4 v = gv[piece];
             uint2* dst = (uint2*)(sv + d * L::V_ROW + kc * 8);
-            dst[0] = make_uint2(v.x, v.y);
-            dst[1] = make_uint2(v.z, v.w);
+            dst[0] = make_uint2(vreg[i][0], vreg[i][1]);
+            dst[1] = make_uint2(vreg[i][2], vreg[i][3]);
         }
         __syncthreads();
+        if (lpage < last_page) AM_LOAD_PAGE(lpage + 1)
         if (!wave_active) continue;
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
@@ -309,27 +326,39 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                 bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(krow + kk * 16));
                 s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], s, 0, 0, 0);
             }
-            float mx = -INFINITY;
+            bool need_mask = !wave_full || key0 + 31 > wave_min_pos || key0 < wave_max_lo;   // wave-uniform
+            if (need_mask) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                int key = key0 + 8 * (e >> 2) + 4 * h2 + (e & 3);
-                float v = (row_ok && key <= my_pos && key >= my_lo) ? s[e] * scale_log2e : -INFINITY;
-                s[e] = v;
-                mx = fmaxf(mx, v);
+                for (int e = 0; e < 16; ++e) {
+                    int key = key0 + 8 * (e >> 2) + 4 * h2 + (e & 3);
+                    s[e] = (row_ok && key <= my_pos && key >= my_lo) ? s[e] : -INFINITY;
+                }
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            float mx = s[0];
+#pragma unroll
+            for (int e = 1; e < 16; ++e) mx = fmaxf(mx, s[e]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * scale_log2e;      // the scale is positive
             float m_new = fmaxf(m, mx);
             float m_use = m_new == -INFINITY ? 0.f : m_new;
-            float corr = fast_exp2(m - m_use);
             float sum = 0.f;
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                s[e] = fast_exp2(s[e] - m_use);
+                s[e] = fast_exp2(fmaf(s[e], scale_log2e, -m_use));
                 sum += s[e];
             }
             sum += __shfl_xor(sum, 32, 64);
-            l = l * corr + sum;
-            m = m_new;
+            // the running maximum rarely moves after the first pieces: rescale only when some
+            // row of the wave needs it
+            if (__builtin_amdgcn_ballot_w64(m_new != m)) {
+                float corr = fast_exp2(m - m_use);
+                l *= corr;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) o[dt][e] *= corr;
+                m = m_new;
+            }
+            l += sum;
             // P^T operands: MFMA u takes elements 8u..8u+7 = keys 16u + {4 h2 .. +3, 8 + 4 h2 .. +3}.
             bf16x8_t pf[2];
 #pragma unroll
@@ -340,8 +369,6 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
-                for (int e = 0; e < 16; ++e) o[dt][e] *= corr;
-#pragma unroll
                 for (int u = 0; u < 2; ++u) {
                     const bf16_t* vrow = sv + (dt * 32 + col) * L::V_ROW + half * 32 + 16 * u + 4 * h2;
                     uint2 a = *(const uint2*)vrow, c = *(const uint2*)(vrow + 8);
@@ -351,6 +378,7 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
             }
         }
     }
+#undef AM_LOAD_PAGE
     if (!row_ok) return;
     float inv = 1.0f / l;
     bf16_t* orow = out + ((size_t)(tok0 + my_row) * hq + h) * D;

@@ -90,7 +90,7 @@ __global__ void rmsnorm_kernel(float* x, const float* __restrict__ gain, TO* __r
 // Same result for rows of up to 8192 values that are a multiple of 4: the row stays in
 // registers between the two passes and all loads are issued at once (a loop of single loads
 // waits for each one in turn, which is what a one-row decode step would spend its time on).
-constexpr int RN_VEC = 8;
+constexpr int RN_MAX_VEC = 8;
 
 __device__ __forceinline__ void store4(float* p, float a, float b, float c, float d) {
     *(float4*)p = make_float4(a, b, c, d);
@@ -102,7 +102,7 @@ __device__ __forceinline__ void store4(bf16_t* p, float a, float b, float c, flo
     *(uint2*)p = v;
 }
 
-template <typename TO>
+template <typename TO, int RN_VEC>
 __global__ void __launch_bounds__(EW_BLOCK)
 rmsnorm_vec_kernel(float* x, const float* __restrict__ gain, TO* __restrict__ out,
                    const int* __restrict__ rows, int n, float eps, const float* __restrict__ partials,
@@ -127,22 +127,24 @@ rmsnorm_vec_kernel(float* x, const float* __restrict__ gain, TO* __restrict__ ou
     if (n_splits > 0) {
         const float4* p4 = (const float4*)(partials + (size_t)src * n);
         long long stride4 = split_stride / 4;
-        for (int sp = 0; sp < n_splits; sp += 2) {      // two splits' loads in flight, added in order
-            bool second = sp + 1 < n_splits;
-            float4 a[RN_VEC], c[RN_VEC];
+        constexpr int GROUP = 32 / RN_VEC;              // splits whose loads are in flight together
+        for (int sp = 0; sp < n_splits; sp += GROUP) {  // loads of a group all issued, added in split order
+            float4 a[GROUP][RN_VEC];
 #pragma unroll
-            for (int j = 0; j < RN_VEC; ++j) {
-                int idx = threadIdx.x + j * EW_BLOCK;
-                int safe = idx < nv ? idx : 0;
-                a[j] = p4[sp * stride4 + safe];
-                c[j] = p4[(second ? sp + 1 : sp) * stride4 + safe];
-            }
+            for (int q = 0; q < GROUP; ++q)
 #pragma unroll
-            for (int j = 0; j < RN_VEC; ++j) {
-                if (threadIdx.x + j * EW_BLOCK >= nv) continue;
-                v[j].x += a[j].x; v[j].y += a[j].y; v[j].z += a[j].z; v[j].w += a[j].w;
-                if (second) { v[j].x += c[j].x; v[j].y += c[j].y; v[j].z += c[j].z; v[j].w += c[j].w; }
-            }
+                for (int j = 0; j < RN_VEC; ++j) {
+                    int idx = threadIdx.x + j * EW_BLOCK;
+                    int safe = idx < nv ? idx : 0;
+                    a[q][j] = p4[(sp + q < n_splits ? sp + q : sp) * stride4 + safe];
+                }
+#pragma unroll
+            for (int q = 0; q < GROUP; ++q)
+#pragma unroll
+                for (int j = 0; j < RN_VEC; ++j) {
+                    if (threadIdx.x + j * EW_BLOCK >= nv || sp + q >= n_splits) continue;
+                    v[j].x += a[q][j].x; v[j].y += a[q][j].y; v[j].z += a[q][j].z; v[j].w += a[q][j].w;
+                }
         }
         if (!rows) {
 #pragma unroll
@@ -174,14 +176,19 @@ ROCML_EXPORT int rocml_rmsnorm(float* x, const float* gain, void* out, int out_d
     ROCML_REQUIRE(n_splits >= 0 && (n_splits == 0 || (partials && split_stride > 0)),
                   "rmsnorm: partial sums need a pointer and a stride");
     if (n_rows == 0) return 0;
-    bool vec = n % 4 == 0 && n <= 4 * RN_VEC * EW_BLOCK && (uintptr_t)x % 16 == 0 &&
+    bool vec = n % 4 == 0 && n <= 4 * RN_MAX_VEC * EW_BLOCK && (uintptr_t)x % 16 == 0 &&
                (uintptr_t)gain % 16 == 0 && (uintptr_t)out % 16 == 0 &&
                (n_splits == 0 || ((uintptr_t)partials % 16 == 0 && split_stride % 4 == 0));
 #define RN_ARGS rows, n, eps, partials, n_splits, split_stride
-    if (vec && out_dtype == ROCML_F32)
-        rmsnorm_vec_kernel<float><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (float*)out, RN_ARGS);
+    bool small = n <= 4 * 4 * EW_BLOCK;      // rows of up to 4096 values: 4 vectors per thread
+    if (vec && out_dtype == ROCML_F32 && small)
+        rmsnorm_vec_kernel<float, 4><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (float*)out, RN_ARGS);
+    else if (vec && out_dtype == ROCML_F32)
+        rmsnorm_vec_kernel<float, 8><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (float*)out, RN_ARGS);
+    else if (vec && out_dtype == ROCML_BF16 && small)
+        rmsnorm_vec_kernel<bf16_t, 4><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (bf16_t*)out, RN_ARGS);
     else if (vec && out_dtype == ROCML_BF16)
-        rmsnorm_vec_kernel<bf16_t><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (bf16_t*)out, RN_ARGS);
+        rmsnorm_vec_kernel<bf16_t, 8><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (bf16_t*)out, RN_ARGS);
     else if (out_dtype == ROCML_F32)
         rmsnorm_kernel<float><<<n_rows, EW_BLOCK, 0, stream>>>(x, gain, (float*)out, RN_ARGS);
     else if (out_dtype == ROCML_BF16)
