@@ -275,7 +275,7 @@ ROCML_EXPORT int rocml_rope_table(const int* pos, const double* inv_freq, float*
 constexpr int QK_MAX_PER_LANE = 8;   // D <= 512
 constexpr int QK_WAVES = EW_BLOCK / WAVE;
 
-template <typename TI, typename TO>
+template <typename TI, typename TO, int QK_PER_LANE>
 __global__ void qk_norm_rope_append_kernel(
     const TI* __restrict__ qkv, int ld, int n_tokens, int hq, int hkv, int d,
     const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
@@ -294,10 +294,10 @@ __global__ void qk_norm_rope_append_kernel(
     int kind = r < hq ? 0 : (r < hq + hkv ? 1 : 2);   // q, k, v
     if (!write_kv && kind != 0) active = false;
     const TI* src = qkv + (size_t)t * ld + (size_t)r * d;
-    float v[QK_MAX_PER_LANE];
+    float v[QK_PER_LANE];
     float ss = 0.f;
 #pragma unroll
-    for (int j = 0; j < QK_MAX_PER_LANE; ++j) {
+    for (int j = 0; j < QK_PER_LANE; ++j) {
         int e = lane + j * WAVE;
         bool ok = active && e < d;
         float val = Elem<TI>::load(ok ? src + e : qkv);
@@ -321,7 +321,7 @@ __global__ void qk_norm_rope_append_kernel(
     if (gain) {
         float inv = 1.0f / sqrtf(wave_sum(ss) / (float)d + eps);
 #pragma unroll
-        for (int j = 0; j < QK_MAX_PER_LANE; ++j) {
+        for (int j = 0; j < QK_PER_LANE; ++j) {
             int e = lane + j * WAVE;
             if (e < d) v[j] = v[j] * inv * gain[e];
         }
@@ -330,7 +330,7 @@ __global__ void qk_norm_rope_append_kernel(
     float* mine = stage + (size_t)wave * d;
     if (rotate) {
 #pragma unroll
-        for (int j = 0; j < QK_MAX_PER_LANE; ++j) {
+        for (int j = 0; j < QK_PER_LANE; ++j) {
             int e = lane + j * WAVE;
             if (e < d) mine[e] = v[j];
         }
@@ -341,7 +341,7 @@ __global__ void qk_norm_rope_append_kernel(
         const float* c = cos_t + (size_t)t * half;
         const float* s = sin_t + (size_t)t * half;
 #pragma unroll
-        for (int j = 0; j < QK_MAX_PER_LANE; ++j) {
+        for (int j = 0; j < QK_PER_LANE; ++j) {
             int e = lane + j * WAVE;
             if (e < rot) {
                 if (e < half) v[j] = v[j] * c[e] - mine[e + half] * s[e];
@@ -362,7 +362,7 @@ __global__ void qk_norm_rope_append_kernel(
             // values are stored transposed inside a page: [page, Hkv, D, page_size]
             TO* vdst = vcache + ((size_t)page * hkv + head) * d * page_size + pos % page_size;
 #pragma unroll
-            for (int j = 0; j < QK_MAX_PER_LANE; ++j) {
+            for (int j = 0; j < QK_PER_LANE; ++j) {
                 int e = lane + j * WAVE;
                 if (e < d) Elem<TO>::store(vdst + (size_t)e * page_size, v[j]);
             }
@@ -371,7 +371,7 @@ __global__ void qk_norm_rope_append_kernel(
         dst = kcache + (((size_t)page * hkv + head) * page_size + pos % page_size) * d;
     }
 #pragma unroll
-    for (int j = 0; j < QK_MAX_PER_LANE; ++j) {
+    for (int j = 0; j < QK_PER_LANE; ++j) {
         int e = lane + j * WAVE;
         if (e < d) Elem<TO>::store(dst + e, v[j]);
     }
@@ -397,16 +397,25 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     long long rows = (long long)n_tokens * (hq + 2 * hkv);
     int grid = ceil_div(rows, QK_WAVES);
     size_t lds = (size_t)QK_WAVES * d * sizeof(float);
-#define LAUNCH(TI, TO)                                                                          \
-    qk_norm_rope_append_kernel<TI, TO><<<grid, EW_BLOCK, lds, stream>>>(                        \
+    int per_lane = d <= 64 ? 1 : d <= 128 ? 2 : d <= 256 ? 4 : 8;     // head values per lane
+#define LAUNCH_N(TI, TO, N)                                                                     \
+    qk_norm_rope_append_kernel<TI, TO, N><<<grid, EW_BLOCK, lds, stream>>>(                     \
         (const TI*)qkv, ld, n_tokens, hq, hkv, d, q_gain, k_gain, eps, cos_t, sin_t, rot,       \
         (TO*)q_out, (TO*)kcache, (TO*)vcache, block_table, bt_width, token_seq, token_pos,      \
         page_size, write_kv, n_splits, split_stride)
-    if (in_dtype == ROCML_F32 && out_dtype == ROCML_F32) LAUNCH(float, float);
-    else if (in_dtype == ROCML_F32 && out_dtype == ROCML_BF16) LAUNCH(float, bf16_t);
-    else if (in_dtype == ROCML_BF16 && out_dtype == ROCML_BF16) LAUNCH(bf16_t, bf16_t);
+#define LAUNCH(TI, TO)                                                                          \
+    {                                                                                           \
+        if (per_lane == 1) LAUNCH_N(TI, TO, 1);                                                 \
+        else if (per_lane == 2) LAUNCH_N(TI, TO, 2);                                            \
+        else if (per_lane == 4) LAUNCH_N(TI, TO, 4);                                            \
+        else LAUNCH_N(TI, TO, 8);                                                               \
+    }
+    if (in_dtype == ROCML_F32 && out_dtype == ROCML_F32) LAUNCH(float, float)
+    else if (in_dtype == ROCML_F32 && out_dtype == ROCML_BF16) LAUNCH(float, bf16_t)
+    else if (in_dtype == ROCML_BF16 && out_dtype == ROCML_BF16) LAUNCH(bf16_t, bf16_t)
     else return rocml_fail("qk_norm_rope_append: unsupported dtype pair in=%d out=%d", in_dtype, out_dtype);
 #undef LAUNCH
+#undef LAUNCH_N
     ROCML_CHECK_LAUNCH("qk_norm_rope_append");
     return 0;
 }

@@ -73,9 +73,10 @@ class Engine:
                 raise RocmlError(f"slot {e.slot} is not a live sequence")
             if len(e.tokens) == 0:
                 raise RocmlError("a step entry needs at least one token")
-            for t in e.tokens:
-                if not 0 <= int(t) < spec.vocab:
-                    raise RocmlError(f"token id {t} is outside the vocabulary of {spec.vocab}")
+            ids = np.asarray(e.tokens, dtype=np.int64)
+            if int(ids.min()) < 0 or int(ids.max()) >= spec.vocab:
+                bad = int(ids[(ids < 0) | (ids >= spec.vocab)][0])
+                raise RocmlError(f"token id {bad} is outside the vocabulary of {spec.vocab}")
             for w in e.want:
                 if not 0 <= int(w) < len(e.tokens):
                     raise RocmlError(f"wanted place {w} is outside the entry's {len(e.tokens)} tokens")

@@ -61,3 +61,55 @@ def test_whole_tail_and_batches(models, name, dtype):
             assert helpers.rel_to_max(got[j], refs[i]) < tol, f"batch order {order}, sequence {i}"
     engine.cache.check()
     assert not engine.cache.lengths
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_internal_cutting_of_long_steps_is_invisible(models, dtype):
+    """A step of more tokens than the engine runs at once is cut into pieces; sequences
+    straddle the cuts and wanted rows come from several pieces."""
+    from rocml_amd.engine import Engine, StepEntry
+    from rocml_amd.weights import load_model
+    path, cfg, weights = models["D"]
+    engine = Engine(load_model(path, dtype=dtype, device="cuda:0"), max_tokens=4096, max_step_tokens=37)
+    oracle_w = _oracle_weights(weights, dtype)
+    prompts = [helpers.random_tokens(n, cfg["vocab_size"], 200 + i) for i, n in enumerate([90, 5, 64, 131])]
+    refs = [plain.forward(cfg, oracle_w, p) for p in prompts]
+    slots = [engine.new_sequence() for _ in prompts]
+    want = [[0, len(p) // 2, len(p) - 1] for p in prompts]
+    logits = engine.step([StepEntry(s, p, w) for s, p, w in zip(slots, prompts, want)]).cpu()
+    expect = torch.cat([ref[w] for ref, w in zip(refs, want)])
+    assert helpers.rel_to_max(logits, expect) < TOL[dtype]
+    # the cache the pieces left is the one a whole step would leave: decode one more token each
+    nxt = [7, 8, 9, 10]
+    logits = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, nxt)]).cpu()
+    expect = torch.stack([plain.forward(cfg, oracle_w, p + [t])[-1] for p, t in zip(prompts, nxt)])
+    assert helpers.rel_to_max(logits, expect) < TOL[dtype]
+    for s in slots:
+        engine.release(s)
+    engine.cache.check()
+
+
+def test_refused_steps_leave_the_engine_as_it_was(models):
+    from rocml_amd.engine import Engine, StepEntry
+    from rocml_amd.errors import CacheFullError, ContextOverflowError, RocmlError
+    from rocml_amd.weights import load_model
+    path, cfg, weights = models["A"]                       # 128 positions
+    engine = Engine(load_model(path, dtype="float32", device="cuda:0"), max_tokens=64 * 2)
+    a, b = engine.new_sequence(), engine.new_sequence()
+    toks = helpers.random_tokens(100, cfg["vocab_size"], 9)
+    ref = plain.forward(cfg, weights, toks)
+    engine.step([StepEntry(a, toks[:60], [])])
+    with pytest.raises(CacheFullError):                    # b would need 2 pages, 1 is free
+        engine.step([StepEntry(b, toks[:], [0]), StepEntry(a, [toks[60]], [0])])
+    with pytest.raises(ContextOverflowError):
+        engine.step([StepEntry(a, helpers.random_tokens(69, cfg["vocab_size"], 1), [0])])
+    with pytest.raises(RocmlError, match="vocabulary"):
+        engine.step([StepEntry(a, [cfg["vocab_size"]], [0])])
+    with pytest.raises(RocmlError, match="twice"):
+        engine.step([StepEntry(a, [1], [0]), StepEntry(a, [2], [0])])
+    with pytest.raises(RocmlError, match="live"):
+        engine.step([StepEntry(17, [1], [0])])
+    assert engine.length(a) == 60 and engine.length(b) == 0
+    engine.cache.check()
+    got = engine.step([StepEntry(a, toks[60:], list(range(40)))]).cpu()    # goes on as if nothing had happened
+    assert helpers.rel_to_max(got, ref[60:]) < TOL["float32"]
