@@ -1,6 +1,6 @@
 """Command line in the manner of the reference's ``rocml-cli`` (rocml-cli/src/main.rs:25-48):
 the subcommands ``generate``, ``bench`` and ``models`` with its option names where it has
-them (rocml-cli/src/common.rs:38-57,146-177; cmd_generate.rs:19-49; cmd_bench.rs:15-77).
+them, plus ``init``, which writes a model folder with random weights, (rocml-cli/src/common.rs:38-57,146-177; cmd_generate.rs:19-49; cmd_bench.rs:15-77).
 Prompts are token ids (``--prompt-ids``); ``--prompt`` takes text when the model folder has a
 ``tokenizer.json``.  There is no chat template, so ``--raw`` is accepted and changes nothing.
 """
@@ -130,6 +130,22 @@ def cmd_models(args) -> int:
     return 0
 
 
+def cmd_init(args) -> int:
+    """Writes a model folder (config.json, model.safetensors) with random weights for a catalog
+    entry or a config.json; the reference has no counterpart (it only reads checkpoints)."""
+    import torch
+    from ..config import read_config_json
+    from ..config.catalog import resolve
+    from ..weights import write_model_dir
+    found = resolve(args.model)
+    config = found.entry.config if found.entry is not None else read_config_json(found.path)
+    jitter = found.entry.init_norm_jitter if found.entry is not None else True
+    dtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
+    path = write_model_dir(args.out, config, args.weights_seed, dtype=dtype, norm_jitter=jitter)
+    print(path)
+    return 0
+
+
 def build_parser() -> argparse.ArgumentParser:
     ap = argparse.ArgumentParser(prog="rocml_amd", description="Qwen3 generation on one MI355X")
     sub = ap.add_subparsers(dest="command", required=True)
@@ -155,6 +171,12 @@ def build_parser() -> argparse.ArgumentParser:
     b.set_defaults(fn=cmd_bench)
     m = sub.add_parser("models", help="list the catalog")
     m.set_defaults(fn=cmd_models)
+    i = sub.add_parser("init", help="write a model folder with random weights")
+    i.add_argument("--model", required=True, help="catalog name, or a folder whose config.json to use")
+    i.add_argument("--out", required=True, help="folder to write config.json and model.safetensors to")
+    i.add_argument("--weights-seed", type=int, default=0)
+    i.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"], help="storage type of the tensors")
+    i.set_defaults(fn=cmd_init)
     return ap
 
 

@@ -33,7 +33,16 @@ TINY_D = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "vocab_s
           "sliding_window": 70,
           "layer_types": ["full_attention", "sliding_attention", "full_attention", "sliding_attention"]}
 
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3)}
+# Sizes that fit none of the fast kernels' rules: a width of 92 and an intermediate size of 150
+# (no multiple of 8), a head size of 112 (a step of 16, no multiple of 32), three query heads on
+# one key/value head, an odd vocabulary.
+TINY_E = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "vocab_size": 257,
+          "hidden_size": 92, "intermediate_size": 150, "num_hidden_layers": 2,
+          "num_attention_heads": 3, "num_key_value_heads": 1, "head_dim": 112,
+          "rope_theta": 1234.5, "rms_norm_eps": 1e-4, "tie_word_embeddings": False,
+          "max_position_embeddings": 300, "hidden_act": "silu", "attention_bias": False}
+
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3), "E": (TINY_E, 4)}
 
 
 def make_model_dir(tmp_path, config: Dict, seed: int, dtype=torch.float32) -> str:

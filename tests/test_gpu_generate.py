@@ -34,7 +34,7 @@ def near_tie(cfg, weights, prompt, produced, k):
     return float((top[0] - top[1]).abs() / top[0].abs().clamp_min(1e-9)) < 1e-2
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_greedy_float32_matches_token_for_token(models, name):
     path, cfg, weights = models[name]
     model = _load(path, "float32", ctx=256, max_batch=3)
