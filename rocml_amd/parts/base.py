@@ -76,8 +76,14 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
+    """What the attention part asks of it: an attribute ``rot_dim`` (the leading width of a head
+    that is rotated, even) and ``tables(step)`` returning ``(cos, sin)``, two 32-bit tensors
+    ``[tokens, rot_dim / 2]`` for the step's ``token_pos``; pair ``(i, i + rot_dim / 2)`` of a
+    head is rotated by the angle whose cosine and sine stand in column ``i``."""
+
     def tables(self, step: Any) -> Any:
-        """Per-step tables for the step's token positions; computed once a step."""
+        """Per-step tables for the step's token positions; computed once a step (``step.memo``
+        is a dictionary that lives as long as the step)."""
         raise NotImplementedError
 
 

@@ -233,3 +233,137 @@ def test_toy_mixer_with_state_registers_builds_and_steps():
     assert helpers.rel_to_max(helpers.run_tail_by_one(engine, b, 10), rb) < 1e-4
     got = helpers.run_batch(engine, [a, b], [30, 3])
     assert helpers.rel_to_max(got[0], ra) < 1e-4 and helpers.rel_to_max(got[1], rb) < 1e-4
+
+
+# ---- a toy feed-forward with routing, and a toy position encoding ---------------------------
+@dataclass(frozen=True)
+class RoutedSpec:
+    hidden: int
+    inter: int
+    n_experts: int
+    top_k: int
+    kind: str = "toy_routed"
+
+
+@dataclass(frozen=True)
+class SlowedRopeSpec:
+    """Rotation whose angle grows with position / factor: the attention part only sees tables."""
+    head_dim: int
+    rot_dim: int
+    theta: float
+    factor: float
+    kind: str = "toy_slowed_rope"
+
+
+def _toy_routed_and_position():
+    from rocml_amd.parts import FeedForward, ParamSpec, PositionEncoding, register_feed_forward, register_position
+
+    class RoutedFfn(FeedForward):
+        """Router logits in 32-bit, the best ``top_k`` experts per token weighted by a softmax over
+        their logits, each expert a small SwiGLU; tokens are gathered per expert."""
+
+        def __init__(self, spec, ctx):
+            self.spec = spec
+
+        def param_specs(self):
+            s = self.spec
+            return {"router.weight": ParamSpec((s.n_experts, s.hidden), role="gain", init="normal"),
+                    "experts.gate_up.weight": ParamSpec((s.n_experts, 2 * s.inter, s.hidden)),
+                    "experts.down.weight": ParamSpec((s.n_experts, s.hidden, s.inter))}
+
+        def bind(self, tensors):
+            self.router = tensors["router.weight"]
+            self.gate_up = tensors["experts.gate_up.weight"].float()
+            self.down = tensors["experts.down.weight"].float()
+
+        def forward(self, step, xn, x_accum):
+            s = self.spec
+            x = xn.float()
+            logits = x @ self.router.t()
+            best, idx = torch.topk(logits, s.top_k, dim=-1)
+            weight = torch.softmax(best, dim=-1)
+            for e in range(s.n_experts):
+                tok, slot = torch.nonzero(idx == e, as_tuple=True)
+                if tok.numel() == 0:
+                    continue
+                gu = x[tok] @ self.gate_up[e].t()
+                h = torch.nn.functional.silu(gu[:, :s.inter]) * gu[:, s.inter:]
+                x_accum.index_add_(0, tok, (h @ self.down[e].t()) * weight[tok, slot][:, None])
+
+    class SlowedRope(PositionEncoding):
+        def __init__(self, spec, ctx):
+            self.spec, self.rot_dim = spec, spec.rot_dim
+            half = spec.rot_dim // 2
+            self.inv = torch.tensor([spec.theta ** (-2.0 * i / spec.rot_dim) for i in range(half)],
+                                    dtype=torch.float64, device=ctx.device)
+
+        def tables(self, step):
+            hit = step.memo.get(("toy_slowed_rope", self.spec))
+            if hit is None:
+                ang = step.token_pos.double()[:, None] / self.spec.factor * self.inv
+                hit = (ang.cos().float().contiguous(), ang.sin().float().contiguous())
+                step.memo[("toy_slowed_rope", self.spec)] = hit
+            return hit
+
+    register_feed_forward("toy_routed", RoutedFfn)
+    register_position("toy_slowed_rope", SlowedRope)
+
+
+def test_toy_routed_feed_forward_and_toy_position_encoding():
+    """Another feed-forward (a router and experts) and another position encoding, defined here and
+    registered: layers 0 and 2 use them, layer 1 is the library's own block."""
+    _toy_routed_and_position()
+    hidden, d = 40, 16
+    slow = SlowedRopeSpec(d, d, 1e4, 4.0)
+    att_slow = AttentionSpec(hidden=hidden, n_heads=4, n_kv_heads=2, head_dim=d, scale=1 / math.sqrt(d), window=None,
+                             qk_norm=NormSpec(d, 1e-5), position=slow)
+    routed = RoutedSpec(hidden, 24, 5, 2)
+
+    def block(mixer, ffn):
+        return BlockSpec(mixer=mixer, ffn=ffn, mixer_norm=NormSpec(hidden, 1e-5), ffn_norm=NormSpec(hidden, 1e-5))
+    layers = [block(att_slow, routed), _block(hidden, _attention_spec(hidden, 4, 2, d)), block(att_slow, routed)]
+    spec = _spec(layers, [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2)], hidden, 83)
+    engine, w = _engine(spec, "float32", seed=8, use_graphs=False)
+
+    def rope_slow(x, positions):
+        return plain.rope_neox(x, [p / slow.factor for p in positions], slow.theta)
+
+    def reference(tokens):
+        x = w["embed.weight"][tokens]
+        pos = list(range(len(tokens)))
+        t = len(tokens)
+        for i, b in enumerate(spec.layers):
+            pre = f"layers.{i}."
+            xn = plain.rmsnorm(x, w[pre + "mixer_norm.weight"], 1e-5)
+            if b.mixer.position.kind == "toy_slowed_rope":
+                m = b.mixer
+                q = plain.rmsnorm((xn @ w[pre + "mixer.q_proj.weight"].t()).reshape(t, m.n_heads, d), w[pre + "mixer.q_norm.weight"], 1e-5)
+                k = plain.rmsnorm((xn @ w[pre + "mixer.k_proj.weight"].t()).reshape(t, m.n_kv_heads, d), w[pre + "mixer.k_norm.weight"], 1e-5)
+                v = (xn @ w[pre + "mixer.v_proj.weight"].t()).reshape(t, m.n_kv_heads, d)
+                o = plain.causal_attention(rope_slow(q, pos), rope_slow(k, pos), v, m.scale, None)
+                x = x + o.reshape(t, -1) @ w[pre + "mixer.o_proj.weight"].t()
+            else:
+                x = x + plain_attention(xn, w, pre + "mixer.", b.mixer, pos)[0]
+            xn = plain.rmsnorm(x, w[pre + "ffn_norm.weight"], 1e-5)
+            if b.ffn.kind == "toy_routed":
+                logits = xn @ w[pre + "ffn.router.weight"].t()
+                out = torch.zeros_like(x)
+                for r in range(t):
+                    best, idx = torch.topk(logits[r], routed.top_k)
+                    wt = torch.softmax(best, -1)
+                    for j in range(routed.top_k):
+                        gu = w[pre + "ffn.experts.gate_up.weight"][idx[j]] @ xn[r]
+                        h = plain.swiglu(gu[:routed.inter], gu[routed.inter:])
+                        out[r] += wt[j] * (w[pre + "ffn.experts.down.weight"][idx[j]] @ h)
+                x = x + out
+            else:
+                x = x + plain.swiglu(xn @ w[pre + "ffn.gate_proj.weight"].t(), xn @ w[pre + "ffn.up_proj.weight"].t()) \
+                    @ w[pre + "ffn.down_proj.weight"].t()
+        return plain.rmsnorm(x, w["final_norm.weight"], 1e-5) @ w["embed.weight"].t()
+
+    a, b = helpers.random_tokens(50, 83, 9), helpers.random_tokens(19, 83, 10)
+    ra, rb = reference(a), reference(b)
+    assert helpers.rel_to_max(helpers.run_whole(engine, a), ra) < 1e-4
+    assert helpers.rel_to_max(helpers.run_tail_by_one(engine, b, 12), rb) < 1e-4
+    got = helpers.run_batch(engine, [a, b], [35, 4])
+    assert helpers.rel_to_max(got[0], ra) < 1e-4 and helpers.rel_to_max(got[1], rb) < 1e-4
