@@ -275,18 +275,20 @@ ROCML_EXPORT int rocml_rope_table(const int* pos, const double* inv_freq, float*
 constexpr int QK_MAX_PER_LANE = 8;   // D <= 512
 constexpr int QK_WAVES = EW_BLOCK / WAVE;
 
-template <typename TI, typename TO, int QK_PER_LANE>
+// LOCAL_PAIR: the whole head is rotated and a lane holds at least two values, so both values of a
+// pair (e, e + d/2) are in the same lane and no exchange through LDS is needed.
+template <typename TI, typename TO, int QK_PER_LANE, bool LOCAL_PAIR>
 __global__ void qk_norm_rope_append_kernel(
     const TI* __restrict__ qkv, int ld, int n_tokens, int hq, int hkv, int d,
     const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot,
     TO* __restrict__ q_out, TO* __restrict__ kcache, TO* __restrict__ vcache,
     const int* __restrict__ block_table, int bt_width, const int* __restrict__ token_seq,
-    const int* __restrict__ token_pos, int page_size, int write_kv, int n_splits, long long split_stride) {
+    const int* __restrict__ token_pos, int page_size, int write_kv, int n_splits, long long split_stride,
+    int rows_per_token) {
     extern __shared__ float stage[];   // [QK_WAVES][d]
     int wave = threadIdx.x / WAVE;
     int lane = threadIdx.x & (WAVE - 1);
-    int rows_per_token = hq + 2 * hkv;
     long long row = (long long)blockIdx.x * QK_WAVES + wave;
     bool active = row < (long long)n_tokens * rows_per_token;
     int t = active ? (int)(row / rows_per_token) : 0;
@@ -327,25 +329,40 @@ __global__ void qk_norm_rope_append_kernel(
         }
     }
     bool rotate = cos_t != nullptr && kind != 2;
-    float* mine = stage + (size_t)wave * d;
-    if (rotate) {
+    if (LOCAL_PAIR) {
+        if (rotate) {
+            constexpr int HJ = QK_PER_LANE / 2 > 0 ? QK_PER_LANE / 2 : 1;
+            const float* c = cos_t + (size_t)t * (d / 2);
+            const float* s = sin_t + (size_t)t * (d / 2);
 #pragma unroll
-        for (int j = 0; j < QK_PER_LANE; ++j) {
-            int e = lane + j * WAVE;
-            if (e < d) mine[e] = v[j];
+            for (int j = 0; j < HJ; ++j) {
+                int e = lane + j * WAVE;                     // pair (e, e + d/2) = values j and j + HJ
+                float cs = c[e], sn = s[e], lo = v[j], hi = v[j + HJ];
+                v[j] = lo * cs - hi * sn;
+                v[j + HJ] = lo * sn + hi * cs;
+            }
         }
-    }
-    __syncthreads();
-    if (rotate) {
-        int half = rot / 2;
-        const float* c = cos_t + (size_t)t * half;
-        const float* s = sin_t + (size_t)t * half;
+    } else {
+        float* mine = stage + (size_t)wave * d;
+        if (rotate) {
 #pragma unroll
-        for (int j = 0; j < QK_PER_LANE; ++j) {
-            int e = lane + j * WAVE;
-            if (e < rot) {
-                if (e < half) v[j] = v[j] * c[e] - mine[e + half] * s[e];
-                else v[j] = mine[e - half] * s[e - half] + v[j] * c[e - half];
+            for (int j = 0; j < QK_PER_LANE; ++j) {
+                int e = lane + j * WAVE;
+                if (e < d) mine[e] = v[j];
+            }
+        }
+        __syncthreads();
+        if (rotate) {
+            int half = rot / 2;
+            const float* c = cos_t + (size_t)t * half;
+            const float* s = sin_t + (size_t)t * half;
+#pragma unroll
+            for (int j = 0; j < QK_PER_LANE; ++j) {
+                int e = lane + j * WAVE;
+                if (e < rot) {
+                    if (e < half) v[j] = v[j] * c[e] - mine[e + half] * s[e];
+                    else v[j] = mine[e - half] * s[e - half] + v[j] * c[e - half];
+                }
             }
         }
     }
@@ -377,6 +394,114 @@ __global__ void qk_norm_rope_append_kernel(
     }
 }
 
+// Prompts: q and k rows of many tokens.  A wave takes ROWS rows and issues the loads of all of
+// them before it works on the first (one row per wave leaves too few bytes in flight and too
+// many tiny blocks to dispatch).  Only the case LOCAL_PAIR describes: whole head rotated, both
+// values of a pair in one lane, complete projections (no partial sums).
+template <typename TI, typename TO, int QK_PER_LANE, int ROWS>
+__global__ void __launch_bounds__(EW_BLOCK)
+qk_norm_rope_rows_kernel(
+    const TI* __restrict__ qkv, int ld, int n_tokens, int hq, int hkv, int d,
+    const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    TO* __restrict__ q_out, TO* __restrict__ kcache, const int* __restrict__ block_table, int bt_width,
+    const int* __restrict__ token_seq, const int* __restrict__ token_pos, int page_size, int rows_per_token) {
+    constexpr int HJ = QK_PER_LANE / 2;
+    int wave = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1);
+    long long total = (long long)n_tokens * rows_per_token;
+    long long row0 = ((long long)blockIdx.x * QK_WAVES + wave) * ROWS;
+    float v[ROWS][QK_PER_LANE], cs[ROWS][HJ], sn[ROWS][HJ];
+    int tok[ROWS], rr[ROWS];
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+        long long row = min(row0 + i, total - 1);            // rows past the end repeat the last one, not stored
+        tok[i] = (int)(row / rows_per_token);
+        rr[i] = (int)(row - (long long)tok[i] * rows_per_token);
+        const TI* src = qkv + (size_t)tok[i] * ld + (size_t)rr[i] * d;
+#pragma unroll
+        for (int j = 0; j < QK_PER_LANE; ++j) v[i][j] = Elem<TI>::load(src + lane + j * WAVE);
+        if (cos_t) {
+#pragma unroll
+            for (int j = 0; j < HJ; ++j) {
+                cs[i][j] = cos_t[(size_t)tok[i] * (d / 2) + lane + j * WAVE];
+                sn[i][j] = sin_t[(size_t)tok[i] * (d / 2) + lane + j * WAVE];
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+        bool is_q = rr[i] < hq;
+        const float* gain = is_q ? q_gain : k_gain;
+        if (gain) {
+            float ss = 0.f;
+#pragma unroll
+            for (int j = 0; j < QK_PER_LANE; ++j) ss = fmaf(v[i][j], v[i][j], ss);
+            float inv = 1.0f / sqrtf(wave_sum(ss) / (float)d + eps);
+#pragma unroll
+            for (int j = 0; j < QK_PER_LANE; ++j) v[i][j] = v[i][j] * inv * gain[lane + j * WAVE];
+        }
+        if (cos_t) {
+#pragma unroll
+            for (int j = 0; j < HJ; ++j) {
+                float lo = v[i][j], hi = v[i][j + HJ];
+                v[i][j] = lo * cs[i][j] - hi * sn[i][j];
+                v[i][j + HJ] = lo * sn[i][j] + hi * cs[i][j];
+            }
+        }
+        if (row0 + i >= total) continue;
+        TO* dst;
+        if (is_q) {
+            dst = q_out + ((size_t)tok[i] * hq + rr[i]) * d;
+        } else {
+            int pos = token_pos[tok[i]];
+            int page = block_table[(size_t)token_seq[tok[i]] * bt_width + pos / page_size];
+            if (page < 0) continue;
+            dst = kcache + (((size_t)page * hkv + (rr[i] - hq)) * page_size + pos % page_size) * d;
+        }
+#pragma unroll
+        for (int j = 0; j < QK_PER_LANE; ++j) Elem<TO>::store(dst + lane + j * WAVE, v[i][j]);
+    }
+}
+
+// Values of many tokens at once (prompts): a block takes 64 consecutive tokens of the packed
+// batch, one key/value head and 32 of its values, stages them in LDS and writes them transposed.
+// In the transposed page a token is one 2- or 4-byte column; written token by token every store
+// would touch a cache line of its own, written this way the 64 lanes of a wave store 64
+// neighbouring positions of one row (they are neighbours wherever the tokens are consecutive
+// positions of one sequence inside one page, which is the rule in a prompt).
+constexpr int VT_TOKENS = 64, VT_VALUES = 32;
+
+template <typename TI, typename TO>
+__global__ void __launch_bounds__(EW_BLOCK)
+v_append_tile_kernel(const TI* __restrict__ qkv, int ld, int n_tokens, int v_col0, int hkv, int d,
+                     TO* __restrict__ vcache, const int* __restrict__ block_table, int bt_width,
+                     const int* __restrict__ token_seq, const int* __restrict__ token_pos, int page_size) {
+    __shared__ float vt_stage[VT_TOKENS][VT_VALUES + 1];
+    int t0 = blockIdx.x * VT_TOKENS, head = blockIdx.y, e0 = blockIdx.z * VT_VALUES;
+    int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+    // thread -> (token tid/32 + 8*i, value tid%32): 128 contiguous bytes per token row
+    float tmp[VT_TOKENS * VT_VALUES / EW_BLOCK];
+#pragma unroll
+    for (int i = 0; i < VT_TOKENS * VT_VALUES / EW_BLOCK; ++i) {
+        int j = min(t0 + (tid >> 5) + (EW_BLOCK / VT_VALUES) * i, n_tokens - 1), e = min(e0 + (tid & 31), d - 1);
+        tmp[i] = Elem<TI>::load(qkv + (size_t)j * ld + v_col0 + (size_t)head * d + e);
+    }
+#pragma unroll
+    for (int i = 0; i < VT_TOKENS * VT_VALUES / EW_BLOCK; ++i) vt_stage[(tid >> 5) + (EW_BLOCK / VT_VALUES) * i][tid & 31] = tmp[i];
+    __syncthreads();
+    int t = t0 + lane;
+    if (t >= n_tokens) return;
+    int pos = token_pos[t];
+    int page = block_table[(size_t)token_seq[t] * bt_width + pos / page_size];
+    if (page < 0) return;
+    TO* dst = vcache + ((size_t)page * hkv + head) * d * page_size + pos % page_size;
+#pragma unroll
+    for (int i = 0; i < VT_VALUES / (EW_BLOCK / WAVE); ++i) {
+        int el = wave + (EW_BLOCK / WAVE) * i;
+        if (e0 + el < d) Elem<TO>::store(dst + (size_t)(e0 + el) * page_size, vt_stage[lane][el]);
+    }
+}
+
 ROCML_EXPORT int rocml_qk_norm_rope_append(
     const void* qkv, int in_dtype, int ld, int n_tokens, int hq, int hkv, int d, const float* q_gain,
     const float* k_gain, float eps, const float* cos_t, const float* sin_t, int rot, void* q_out,
@@ -394,21 +519,41 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     ROCML_REQUIRE(!write_kv || (page_size > 0 && bt_width > 0 && block_table && kcache && vcache),
                   "qk_norm_rope_append: cache arguments missing");
     if (n_tokens == 0) return 0;
-    long long rows = (long long)n_tokens * (hq + 2 * hkv);
-    int grid = ceil_div(rows, QK_WAVES);
-    size_t lds = (size_t)QK_WAVES * d * sizeof(float);
+    // prompts: the values go through the transposing tile kernel, the row kernel does q and k
+    bool v_tiled = write_kv && n_splits == 1 && n_tokens >= VT_TOKENS;
+    int rows_per_token = hq + (write_kv ? (v_tiled ? hkv : 2 * hkv) : 0);
+    long long rows = (long long)n_tokens * rows_per_token;
     int per_lane = d <= 64 ? 1 : d <= 128 ? 2 : d <= 256 ? 4 : 8;     // head values per lane
-#define LAUNCH_N(TI, TO, N)                                                                     \
-    qk_norm_rope_append_kernel<TI, TO, N><<<grid, EW_BLOCK, lds, stream>>>(                     \
+    // both values of a rotation pair in one lane: whole head rotated, d = per_lane * 64
+    bool local_pair = per_lane >= 2 && (rot == d || rot == 0) && d == per_lane * WAVE;
+    // many rows, none of them values: several rows per wave
+    bool many_rows = local_pair && per_lane <= 4 && n_splits == 1 && n_tokens >= VT_TOKENS && (v_tiled || !write_kv);
+    constexpr int MANY = 4;
+    int grid = many_rows ? ceil_div(rows, QK_WAVES * MANY) : ceil_div(rows, QK_WAVES);
+    size_t lds = local_pair ? 0 : (size_t)QK_WAVES * d * sizeof(float);
+#define LAUNCH_N(TI, TO, N, LP)                                                                 \
+    qk_norm_rope_append_kernel<TI, TO, N, LP><<<grid, EW_BLOCK, lds, stream>>>(                 \
         (const TI*)qkv, ld, n_tokens, hq, hkv, d, q_gain, k_gain, eps, cos_t, sin_t, rot,       \
         (TO*)q_out, (TO*)kcache, (TO*)vcache, block_table, bt_width, token_seq, token_pos,      \
-        page_size, write_kv, n_splits, split_stride)
+        page_size, write_kv, n_splits, split_stride, rows_per_token)
+#define LAUNCH_ROWS(TI, TO, N)                                                                  \
+    qk_norm_rope_rows_kernel<TI, TO, N, MANY><<<grid, EW_BLOCK, 0, stream>>>(                   \
+        (const TI*)qkv, ld, n_tokens, hq, hkv, d, q_gain, k_gain, eps, rot ? cos_t : nullptr,   \
+        rot ? sin_t : nullptr, (TO*)q_out, (TO*)kcache, block_table, bt_width, token_seq,       \
+        token_pos, page_size, rows_per_token)
 #define LAUNCH(TI, TO)                                                                          \
     {                                                                                           \
-        if (per_lane == 1) LAUNCH_N(TI, TO, 1);                                                 \
-        else if (per_lane == 2) LAUNCH_N(TI, TO, 2);                                            \
-        else if (per_lane == 4) LAUNCH_N(TI, TO, 4);                                            \
-        else LAUNCH_N(TI, TO, 8);                                                               \
+        if (many_rows) { if (per_lane == 2) LAUNCH_ROWS(TI, TO, 2); else LAUNCH_ROWS(TI, TO, 4); } \
+        else if (per_lane == 1) LAUNCH_N(TI, TO, 1, false);                                     \
+        else if (per_lane == 2) { if (local_pair) LAUNCH_N(TI, TO, 2, true); else LAUNCH_N(TI, TO, 2, false); } \
+        else if (per_lane == 4) { if (local_pair) LAUNCH_N(TI, TO, 4, true); else LAUNCH_N(TI, TO, 4, false); } \
+        else { if (local_pair) LAUNCH_N(TI, TO, 8, true); else LAUNCH_N(TI, TO, 8, false); }    \
+        if (v_tiled) {                                                                          \
+            dim3 vgrid(ceil_div(n_tokens, VT_TOKENS), hkv, ceil_div(d, VT_VALUES));             \
+            v_append_tile_kernel<TI, TO><<<vgrid, EW_BLOCK, 0, stream>>>(                       \
+                (const TI*)qkv, ld, n_tokens, (hq + hkv) * d, hkv, d, (TO*)vcache, block_table, \
+                bt_width, token_seq, token_pos, page_size);                                     \
+        }                                                                                       \
     }
     if (in_dtype == ROCML_F32 && out_dtype == ROCML_F32) LAUNCH(float, float)
     else if (in_dtype == ROCML_F32 && out_dtype == ROCML_BF16) LAUNCH(float, bf16_t)
@@ -416,6 +561,7 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     else return rocml_fail("qk_norm_rope_append: unsupported dtype pair in=%d out=%d", in_dtype, out_dtype);
 #undef LAUNCH
 #undef LAUNCH_N
+#undef LAUNCH_ROWS
     ROCML_CHECK_LAUNCH("qk_norm_rope_append");
     return 0;
 }

@@ -37,18 +37,23 @@ static int launch_mfma_tile_as(const void* x, int ldx, const void* w, int ldw, v
     return 0;
 }
 
-// big: 0 = choose, 1 = 128x128 tiles, 2 = 256x256 tiles.  Measured on large products the big
-// tile reaches about 975 TFLOP/s and the small one about 800, but a CU holds one big tile or
-// two small ones at a time, and the last round of tiles may leave CUs idle: the choice weighs
-// the speed with the share of the 256 CUs that the rounds keep busy.
+// shape: 0 = choose, 1 = 128x128 tiles, 2 = 256x256.  Measured in the model (weights from HBM)
+// the big tile reaches about 1030 TFLOP/s on products that fill the chip and the small one
+// about 760 (the wider a wave's own tile and the more waves share an operand, the fewer LDS
+// bytes per product), but a CU holds one big tile or two small ones at a time, and the last
+// round of tiles may leave CUs idle: the choice weighs the speed with the share of the 256 CUs
+// that the rounds keep busy.
 template <int EPI>
 static int launch_mfma_tile(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m,
-                            int n, int k, int big, hipStream_t stream) {
-    double t256 = (double)ceil_div(m, 256) * ceil_div(n, 256), t128 = (double)ceil_div(m, 128) * ceil_div(n, 128);
-    double score256 = 975.0 * t256 / (ceil_div((long long)t256, 256) * 256.0);
-    double score128 = 800.0 * t128 / (ceil_div((long long)t128, 512) * 512.0);
-    bool use256 = big == 2 || (big == 0 && score256 > score128);
-    if (use256) return launch_mfma_tile_as<EPI, GemmTile256>(x, ldx, w, ldw, out, ldo, m, n, k, stream);
+                            int n, int k, int shape, hipStream_t stream) {
+    if (shape == 0) {
+        auto fill = [&](int bm, int bn, int per_round) {
+            double tiles = (double)ceil_div(m, bm) * ceil_div(n, bn);
+            return tiles / (ceil_div((long long)tiles, per_round) * (double)per_round);
+        };
+        shape = 1030.0 * fill(256, 256, 256) > 760.0 * fill(128, 128, 512) ? 2 : 1;
+    }
+    if (shape == 2) return launch_mfma_tile_as<EPI, GemmTile256>(x, ldx, w, ldw, out, ldo, m, n, k, stream);
     return launch_mfma_tile_as<EPI, GemmTile128>(x, ldx, w, ldw, out, ldo, m, n, k, stream);
 }
 

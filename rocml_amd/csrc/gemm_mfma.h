@@ -2,14 +2,15 @@
 // 32-bit accumulation.  Both operands are K-contiguous, which is what an MFMA lane wants: 8
 // consecutive K values (16 bytes) of one row.
 //
-// Two kernels:
-//  * gemm_mfma_kernel, many rows (prefill): 128x128 output tile per 256-thread block, four
-//    waves in 2x2, each wave 64x64 = 2x2 tiles of v_mfma_f32_32x32x16_bf16; K staged 64 at a
-//    time through double-buffered LDS with one barrier per stage; rows padded by 16 bytes so
-//    that 128-bit LDS reads of 16 rows fall into 16 different bank groups.  The idea of the
-//    tiling (big tile per block, 2x2 fragments per wave, padded double-buffered LDS) is the
-//    reference's WMMA kernel (rocml-kernels/kernels/gemm_xwt_wmma_impl.h:211-378); layouts and
-//    sizes are for wave64 MFMA.  Blocks are renumbered so that each of the 8 XCDs works on a
+// Kernels:
+//  * gemm_mfma_kernel, many rows (prefill): an output tile per block, each wave a grid of
+//    v_mfma_f32_32x32x16_bf16 tiles (128x64 per wave in the 256-wide shapes, 64x64 in the
+//    128x128 one); K staged 64 at a time through double-buffered LDS with one barrier per stage;
+//    rows padded by 16 bytes so that 128-bit LDS reads of 16 rows fall into 16 different bank
+//    groups.  The idea of the tiling (big tile per block, a grid of fragments per wave, padded
+//    double-buffered LDS) is the reference's WMMA kernel
+//    (rocml-kernels/kernels/gemm_xwt_wmma_impl.h:211-378); layouts, sizes and the instruction
+//    schedule are for wave64 MFMA.  Blocks are renumbered so that each of the 8 XCDs works on a
 //    contiguous range of tiles and its L2 sees few weight panels.
 //  * gemm_skinny_kernel, few rows (decode, M <= 64): memory-bound; a block owns 64 weight rows
 //    and a K range, each wave 16 rows.  Weights go straight from global memory into MFMA
@@ -55,9 +56,12 @@ __device__ __forceinline__ void epilogue_store(void* out, size_t idx, float v) {
 }
 
 // ---- many rows ---------------------------------------------------------------------------
-// One kernel, two shapes (see GemmTile below): 128x128 with four waves for most products, and
-// 256x256 with eight waves (two per SIMD, each 128x64) for products wide enough to give every
-// CU several such tiles: four times the products per LDS byte and per barrier.
+// One kernel, two shapes (see GemmTile below): 256x256 with eight waves (two per SIMD, each
+// 128x64) for products wide enough to give every CU such a tile, 128x128 with four waves of
+// 64x64 (two blocks per CU) for the rest.  (256x128 with four waves of 128x64 was tried: one
+// wave per SIMD has nobody to cover for it while it waits for weights from HBM.  Reading four
+// bytes of every row's line some stages ahead, to pull it into L2, was tried too: the extra
+// requests cost more than the earlier arrival gains.)
 constexpr int GM_BK = 64;
 constexpr int GM_ROW = GM_BK / 8 + 1;                 // u32x4_t per LDS row, one of padding
 
@@ -72,7 +76,7 @@ struct GemmTile {
     static constexpr int LDS_BYTES = 2 * (BM + BN) * GM_ROW * 16;   // two stages
 };
 using GemmTile128 = GemmTile<2, 2, 2, 2>;
-using GemmTile256 = GemmTile<2, 4, 4, 2>;
+using GemmTile256 = GemmTile<2, 4, 4, 2>;       // eight waves (two per SIMD), 128x64 each
 
 template <int EPI, typename T>
 __global__ void __launch_bounds__(T::THREADS)
@@ -80,6 +84,15 @@ gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
                  void* __restrict__ out, int ldo, int m, int n, int k, int tiles_m, int n_tiles) {
     extern __shared__ u32x4_t gm_smem[];              // [2 stages][A: BM rows | B: BN rows][GM_ROW]
     constexpr int STAGE = (T::BM + T::BN) * GM_ROW;
+    constexpr int NREG = T::PA + T::PB;               // 16-byte pieces a thread moves per K stage
+    constexpr int PROD = T::TM * T::TN;               // products per 16-wide K slice
+    constexpr int KK = GM_BK / 16;                    // slices per stage
+    static_assert(KK == 4, "the schedule below is written for four slices per stage");
+    // piece r is stored after product r * 2*PROD / NREG of the first two slices; its register is
+    // refilled one product later when every store has a free product behind it, else at the same
+    // place in the last two slices
+    static_assert(2 * PROD >= NREG, "the stores must fit into the first two slices");
+    constexpr bool REFILL_AT_ONCE = 2 * PROD >= 2 * NREG;
     int per_xcd = gridDim.x / 8;
     int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
     if (logical >= n_tiles) return;
@@ -88,11 +101,6 @@ gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
     int wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;
     int lrow = tid >> 3, lkc = tid & 7;
     int nk = (k + GM_BK - 1) / GM_BK;
-    // The global loads of the next K stage are issued before the current stage is multiplied
-    // and written to the other LDS buffer afterwards: one barrier per stage.  (Loading two
-    // stages ahead was tried: the compiler then keeps two sets of accumulators and the kernel
-    // is slower.)
-    u32x4_t ra[T::PA], rb[T::PB];
     f32x16_t acc[T::TM][T::TN];
 #pragma unroll
     for (int i = 0; i < T::TM; ++i)
@@ -101,70 +109,93 @@ gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
+    // Schedule of one K stage (64 wide = four slices of 16), written out by hand and pinned with
+    // scheduling barriers, because left alone the compiler sinks every LDS read to its first use
+    // and gathers the stores behind the products:
+    //  * the operand pieces of the next slice are read from LDS before the products of the
+    //    current slice are issued (two register sets);
+    //  * the pieces of the next stage, loaded from global memory one stage ago, are stored to the
+    //    other LDS buffer between the products of slices 0 and 1, and each register is refilled
+    //    from the stage after that: the memory pipes work while the matrix core does, and a load
+    //    has a whole stage to arrive;
+    //  * the one barrier of a stage stands after slice 2.  By then every wave has stored its
+    //    pieces of the next stage and has read the last pieces of this one, so during slice 3 the
+    //    first operands of the next stage are fetched and the matrix core does not wait for LDS
+    //    when the stage changes.
     // Loads go to clamped addresses and are used as they come: rows beyond M or N only feed
-    // outputs that are never stored.  Only a 16-byte piece beyond K must count as zero, and that
-    // is decided when the piece is written to LDS, long after the load was issued (a select
-    // right behind the load would make the wave wait for it there).
-    const bf16_t* xrow[T::PA];
-    const bf16_t* wrow[T::PB];
+    // outputs that are never stored, and a piece beyond K is zeroed when it is stored to LDS.
+    // Nothing in the loop is conditional, so the count of outstanding loads is known at every
+    // wait; the last stages load and store pieces nobody reads.
+    u32x4_t reg[NREG];
+    const bf16_t* src[NREG];
+    int dst[NREG];                                    // LDS index of the piece within a stage
 #pragma unroll
-    for (int i = 0; i < T::PA; ++i) xrow[i] = x + (size_t)min(m0 + lrow + T::PASS_ROWS * i, m - 1) * ldx;
-#pragma unroll
-    for (int i = 0; i < T::PB; ++i) wrow[i] = w + (size_t)min(n0 + lrow + T::PASS_ROWS * i, n - 1) * ldw;
-    // Written as macros over the register arrays: handed to a function through a pointer, the
-    // arrays would be kept in scratch memory and every load waited for at once.
-#define GM_LOAD_GLOBAL(kt_)                                                                      \
-    {                                                                                            \
-        int gk_ = (kt_) * GM_BK + lkc * 8;                                                       \
-        gk_ = gk_ < k ? gk_ : 0;                                                                 \
-        _Pragma("unroll") for (int i = 0; i < T::PA; ++i) ra[i] = *(const u32x4_t*)(xrow[i] + gk_); \
-        _Pragma("unroll") for (int i = 0; i < T::PB; ++i) rb[i] = *(const u32x4_t*)(wrow[i] + gk_); \
+    for (int r = 0; r < NREG; ++r) {
+        bool is_a = r < T::PA;
+        int row = lrow + T::PASS_ROWS * (is_a ? r : r - T::PA);
+        src[r] = is_a ? x + (size_t)min(m0 + row, m - 1) * ldx + lkc * 8
+                      : w + (size_t)min(n0 + row, n - 1) * ldw + lkc * 8;
+        dst[r] = (is_a ? 0 : T::BM * GM_ROW) + row * GM_ROW + lkc;
     }
-#define GM_STORE_LDS(kt_, buf_)                                                                  \
-    {                                                                                            \
-        u32x4_t* sa_ = gm_smem + (buf_) * STAGE;                                                 \
-        u32x4_t* sb_ = sa_ + T::BM * GM_ROW;                                                     \
-        bool kin_ = (kt_) * GM_BK + lkc * 8 < k;                                                 \
-        const u32x4_t zero_ = {0u, 0u, 0u, 0u};                                                  \
-        _Pragma("unroll") for (int i = 0; i < T::PA; ++i)                                        \
-            sa_[(lrow + T::PASS_ROWS * i) * GM_ROW + lkc] = kin_ ? ra[i] : zero_;                \
-        _Pragma("unroll") for (int i = 0; i < T::PB; ++i)                                        \
-            sb_[(lrow + T::PASS_ROWS * i) * GM_ROW + lkc] = kin_ ? rb[i] : zero_;                \
+    const u32x4_t zero = {0u, 0u, 0u, 0u};
+    int fa = (wm * T::TM * 32 + (lane & 31)) * GM_ROW + (lane >> 5);
+    int fb = T::BM * GM_ROW + (wn * T::TN * 32 + (lane & 31)) * GM_ROW + (lane >> 5);
+    // offset of this thread's piece in stage kt, or back to the row's start when it is beyond K
+#define GM_KOFF(kt_) ((kt_) * GM_BK + lkc * 8 < k ? (kt_) * GM_BK : -lkc * 8)
+    {
+        int o0 = GM_KOFF(0);
+        bool in0 = lkc * 8 < k;
+#pragma unroll
+        for (int r = 0; r < NREG; ++r) reg[r] = *(const u32x4_t*)(src[r] + o0);
+#pragma unroll
+        for (int r = 0; r < NREG; ++r) gm_smem[dst[r]] = in0 ? reg[r] : zero;
+        int o1 = GM_KOFF(1);
+#pragma unroll
+        for (int r = 0; r < NREG; ++r) reg[r] = *(const u32x4_t*)(src[r] + o1);
     }
-    auto multiply = [&](int buf) {
-        const u32x4_t* sa = gm_smem + buf * STAGE;
-        const u32x4_t* sb = sa + T::BM * GM_ROW;
-#pragma unroll
-        for (int kk = 0; kk < GM_BK / 16; ++kk) {
-            bf16x8_t a[T::TM], b[T::TN];
-            int col = kk * 2 + (lane >> 5);
-#pragma unroll
-            for (int i = 0; i < T::TM; ++i)
-                a[i] = as_frag4(sa[(wm * T::TM * 32 + i * 32 + (lane & 31)) * GM_ROW + col]);
-#pragma unroll
-            for (int j = 0; j < T::TN; ++j)
-                b[j] = as_frag4(sb[(wn * T::TN * 32 + j * 32 + (lane & 31)) * GM_ROW + col]);
-#pragma unroll
-            for (int i = 0; i < T::TM; ++i)
-#pragma unroll
-                for (int j = 0; j < T::TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
-        }
-    };
-
-    GM_LOAD_GLOBAL(0)
-    GM_STORE_LDS(0, 0)
     __syncthreads();
+    bf16x8_t a[2][T::TM], b[2][T::TN];
+#pragma unroll
+    for (int i = 0; i < T::TM; ++i) a[0][i] = as_frag4(gm_smem[fa + i * 32 * GM_ROW]);
+#pragma unroll
+    for (int j = 0; j < T::TN; ++j) b[0][j] = as_frag4(gm_smem[fb + j * 32 * GM_ROW]);
     for (int kt = 0; kt < nk; ++kt) {
-        int buf = kt & 1;
-        bool more = kt + 1 < nk;
-        if (more) GM_LOAD_GLOBAL(kt + 1)
-        multiply(buf);
-        if (more) GM_STORE_LDS(kt + 1, buf ^ 1)
-        __syncthreads();
+        const u32x4_t* cur = gm_smem + (kt & 1) * STAGE;
+        u32x4_t* nxt = gm_smem + ((kt + 1) & 1) * STAGE;
+        bool in1 = (kt + 1) * GM_BK + lkc * 8 < k;    // is the piece held in registers inside K
+        int o2 = GM_KOFF(kt + 2);
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            int c = kk & 1;
+            const u32x4_t* from = kk + 1 < KK ? cur + (kk + 1) * 2 : nxt;   // slice 3 fetches the next stage's slice 0
+#pragma unroll
+            for (int i = 0; i < T::TM; ++i) a[c ^ 1][i] = as_frag4(from[fa + i * 32 * GM_ROW]);
+#pragma unroll
+            for (int j = 0; j < T::TN; ++j) b[c ^ 1][j] = as_frag4(from[fb + j * 32 * GM_ROW]);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int q = 0; q < PROD; ++q) {
+                acc[q / T::TN][q % T::TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                    a[c][q / T::TN], b[c][q % T::TN], acc[q / T::TN][q % T::TN], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                // the piece whose place is product s of a half stage: r with r * 2*PROD / NREG == s
+                int half_slot = (kk & 1) * PROD + q;
+                int r = (half_slot * NREG + 2 * PROD - 1) / (2 * PROD);
+                bool here = r < NREG && r * 2 * PROD / NREG == half_slot;
+                int rp = ((half_slot - 1) * NREG + 2 * PROD - 1) / (2 * PROD);      // the piece one product earlier
+                bool before = half_slot >= 1 && rp < NREG && rp * 2 * PROD / NREG == half_slot - 1;
+                if (kk < 2) {
+                    if (here) nxt[dst[r]] = in1 ? reg[r] : zero;
+                    else if (REFILL_AT_ONCE && before) reg[rp] = *(const u32x4_t*)(src[rp] + o2);
+                } else if (!REFILL_AT_ONCE && here) {
+                    reg[r] = *(const u32x4_t*)(src[r] + o2);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (kk == 2) __syncthreads();
+        }
     }
-#undef GM_LOAD_GLOBAL
-#undef GM_STORE_LDS
+#undef GM_KOFF
     // Accumulator element e of a lane: row 8*(e/4) + 4*(lane/32) + e%4, column lane%32.
 #pragma unroll
     for (int i = 0; i < T::TM; ++i)

@@ -143,7 +143,9 @@ def _qkv_case(tokens, hq, hkv, d, pos_base, theta, rot, norm, dtype, seed=0, spl
 
 @pytest.mark.parametrize("tokens,hq,hkv,d,pos_base,rot,norm", [
     (10, 3, 3, 16, 5, 16, True), (1, 2, 1, 4, 0, 4, True), (70, 4, 2, 48, 100, 48, True),
-    (5, 2, 2, 128, 60, 64, True), (5, 6, 2, 32, 0, 32, False), (3, 2, 1, 16, 7, 0, True), (2, 1, 1, 264, 1, 264, True)])
+    (5, 2, 2, 128, 60, 64, True), (5, 6, 2, 32, 0, 32, False), (3, 2, 1, 16, 7, 0, True), (2, 1, 1, 264, 1, 264, True),
+    # whole head rotated with both values of a pair in one lane; many tokens: values through the transposing kernel
+    (3, 8, 2, 128, 60, 128, True), (150, 4, 2, 128, 37, 128, True), (64, 2, 1, 256, 0, 256, True), (129, 2, 2, 80, 63, 80, False)])
 def test_qk_norm_rope_append(tokens, hq, hkv, d, pos_base, rot, norm):
     gq, gk, gv, q, k, v, (kc, vc, table, positions) = _qkv_case(tokens, hq, hkv, d, pos_base, 1e4, rot, norm, torch.float32)
     assert float((gq - q).abs().max()) < 1e-5
@@ -153,7 +155,8 @@ def test_qk_norm_rope_append(tokens, hq, hkv, d, pos_base, rot, norm):
     written = torch.zeros(kc.shape[0], 64, dtype=torch.bool)
     for p in positions:
         written[table[0, p // 64], p % 64] = True
-    assert float(kc.cpu()[~written.unsqueeze(1).expand(-1, kc.shape[1], -1)].abs().max()) == 0.0
+    assert float(kc.cpu()[~written.unsqueeze(1).expand(-1, kc.shape[1], -1)].abs().sum()) == 0.0
+    assert float(vc.cpu().transpose(2, 3)[~written.unsqueeze(1).expand(-1, vc.shape[1], -1)].abs().sum()) == 0.0
     gq, gk, gv, *_ = _qkv_case(tokens, hq, hkv, d, pos_base, 1e4, rot, norm, torch.bfloat16)
     assert float((gq - q).abs().max()) < 8e-3 * float(q.abs().max())
     assert float((gk - k).abs().max()) < 8e-3 * float(k.abs().max())
