@@ -63,17 +63,27 @@ template <int MT, int EPI>
 static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m, int n,
                          int k, void* workspace, long long workspace_bytes, SplitPlan plan, hipStream_t stream) {
     constexpr int LDS = 2 * MT * 16 * GS_ROW * 16;
+    // Waves per block.  The activations of a K chunk take LDS in proportion to the rows, and LDS
+    // decides how many blocks a CU holds: with 64 rows two.  Eight waves per block then double
+    // the weight bytes in flight per CU and halve the times the activations are read.  One row
+    // tile without a split (wide products) gets two waves: more, smaller blocks keep more loads
+    // in flight when nothing else multiplies their number.
+    constexpr int WIDE = MT == 4 ? 8 : 4;
+    constexpr bool CAN_NARROW = MT == 1;
+    constexpr bool DEEP = MT == 4;                    // weights two chunks ahead (gemm_skinny_deep_kernel)
     static bool ready = false;
     if (!ready) {
-        if (allow_lds(gemm_skinny_kernel<MT, EPI, false>, LDS, "gemm")) return 1;
-        if (allow_lds(gemm_skinny_kernel<MT, EPI, true>, LDS, "gemm")) return 1;
+        if constexpr (DEEP) {
+            if (allow_lds(gemm_skinny_deep_kernel<MT, EPI, false, WIDE>, LDS, "gemm")) return 1;
+            if (allow_lds(gemm_skinny_deep_kernel<MT, EPI, true, WIDE>, LDS, "gemm")) return 1;
+        } else {
+            if (allow_lds(gemm_skinny_kernel<MT, EPI, false, WIDE>, LDS, "gemm")) return 1;
+            if (allow_lds(gemm_skinny_kernel<MT, EPI, true, WIDE>, LDS, "gemm")) return 1;
+        }
         ready = true;
     }
-    // Wide products without a split get blocks of two waves: more, smaller blocks keep more
-    // loads in flight when nothing else multiplies their number.
-    constexpr bool CAN_NARROW = MT == 1;
     bool narrow = CAN_NARROW && (EPI == EPI_SWIGLU || n >= 65536);
-    int blocks_n = ceil_div(n, narrow ? 32 : GS_BN);
+    int blocks_n = ceil_div(n, narrow ? 32 : 16 * WIDE);
     int target = MT == 4 ? 256 : 512;
     int splits = target / blocks_n;
     int by_k = k / 512;
@@ -92,11 +102,19 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
             gemm_skinny_kernel<MT, EPI, false, 2><<<grid, 128, LDS, stream>>>(
                 (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
     } else if (splits == 1) {
-        gemm_skinny_kernel<MT, EPI, false><<<grid, GS_THREADS, LDS, stream>>>(
-            (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
+        if constexpr (DEEP)
+            gemm_skinny_deep_kernel<MT, EPI, false, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
+                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
+        else
+            gemm_skinny_kernel<MT, EPI, false, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
+                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
     } else {
-        gemm_skinny_kernel<MT, EPI, true><<<grid, GS_THREADS, LDS, stream>>>(
-            (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, workspace, n, m, n, k, k_per_split);
+        if constexpr (DEEP)
+            gemm_skinny_deep_kernel<MT, EPI, true, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
+                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, workspace, n, m, n, k, k_per_split);
+        else
+            gemm_skinny_kernel<MT, EPI, true, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
+                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, workspace, n, m, n, k, k_per_split);
         if (plan.defer && ldo == n) {
             // the caller's next kernel adds the partial sums itself
             *plan.deferred = splits;

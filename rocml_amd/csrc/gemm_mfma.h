@@ -12,12 +12,16 @@
 //    (rocml-kernels/kernels/gemm_xwt_wmma_impl.h:211-378); layouts, sizes and the instruction
 //    schedule are for wave64 MFMA.  Blocks are renumbered so that each of the 8 XCDs works on a
 //    contiguous range of tiles and its L2 sees few weight panels.
-//  * gemm_skinny_kernel, few rows (decode, M <= 64): memory-bound; a block owns 64 weight rows
-//    and a K range, each wave 16 rows.  Weights go straight from global memory into MFMA
-//    operand registers (v_mfma_f32_16x16x32_bf16), 8 loads of 16 bytes in flight per lane; the
+//  * gemm_skinny_kernel, few rows (decode, M <= 64): memory-bound; a block owns 16 weight rows
+//    per wave and a K range.  Weights go straight from global memory into MFMA operand
+//    registers (v_mfma_f32_16x16x32_bf16), 8 loads of 16 bytes in flight per lane; the
 //    activations of the K range are shared through LDS.  Split-K partial sums go to a
-//    workspace and are added in split order by a second kernel, so results do not depend on
-//    timing (rocml-kernels/kernels/gemm_splitk_reduce.hip:4-10 has the same rule).
+//    workspace and are added in split order by a second kernel (or by the caller's next
+//    kernel), so results do not depend on timing
+//    (rocml-kernels/kernels/gemm_splitk_reduce.hip:4-10 has the same rule).
+//    gemm_skinny_deep_kernel is the same with weights requested two chunks ahead, for blocks
+//    of 64 rows.
+//  * gemm_kpar_kernel, one or two rows: the waves of a block split K and meet once in LDS.
 #pragma once
 #include "common.h"
 
@@ -221,6 +225,34 @@ gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
 constexpr int GS_BN = 64, GS_KC = 256, GS_THREADS = 256;
 constexpr int GS_ROW = GS_KC / 8 + 1;                 // uint4 per LDS row of activations
 
+// Accumulator element e of a lane: weight row (lane/16)*4 + e, activation row lane%16.
+template <int MT, int EPI, bool PARTIAL>
+__device__ __forceinline__ void skinny_epilogue(const f32x4_t (&acc)[MT], void* out, int ldo, int m, int n, int n0,
+                                                int lane, int split) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        int gm = mt * 16 + (lane & 15);
+        if (gm >= m) continue;
+        if (EPI == EPI_SWIGLU && !PARTIAL) {
+            // a lane holds weight rows 4g .. 4g+3 = two (gate, up) pairs
+#pragma unroll
+            for (int e = 0; e < 4; e += 2) {
+                int gn = n0 + (lane >> 4) * 4 + e;
+                if (gn + 1 < n)
+                    ((bf16_t*)out)[(size_t)gm * ldo + (gn >> 1)] = f32_to_bf16(silu_mul(acc[mt][e], acc[mt][e + 1]));
+            }
+            continue;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            int gn = n0 + (lane >> 4) * 4 + e;
+            if (gn >= n) continue;
+            if (PARTIAL) ((float*)out)[((size_t)split * m + gm) * n + gn] = acc[mt][e];
+            else epilogue_store<EPI>(out, (size_t)gm * ldo + gn, acc[mt][e]);
+        }
+    }
+}
+
 // PARTIAL: write 32-bit partial sums [split][M][N] instead of the epilogue.
 // Loads are never followed by a select: addresses beyond the matrix are clamped to a place
 // inside it, rows beyond M or N only feed outputs that are not stored, and a piece beyond K is
@@ -313,29 +345,115 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restri
 #undef GS_LOAD_W
 #undef GS_LOAD_X
 #undef GS_STORE_X
-    // Accumulator element e of a lane: weight row (lane/16)*4 + e, activation row lane%16.
+    skinny_epilogue<MT, EPI, PARTIAL>(acc, out, ldo, m, n, n0, lane, blockIdx.y);
+}
+
+// The same product for blocks of 64 rows, where the chip holds few waves (LDS for the
+// activations limits a CU to two blocks): weights are requested two chunks ahead instead of one,
+// so that a wave always has 8 to 16 loads of 16 bytes outstanding.  (For fewer rows, with four
+// times the blocks per CU, the deeper pipeline only lengthens the start and was slower.)
+template <int MT, int EPI, bool PARTIAL, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES)
+gemm_skinny_deep_kernel(const bf16_t* x, int ldx, const bf16_t* w, int ldw,
+                   void* out, int ldo, int m, int n, int k, int k_per_split) {
+    // (no __restrict__: a load from memory that is promised not to change may be moved anywhere,
+    // and the order of the loads below is the point)
+    extern __shared__ u32x4_t gs_smem[];              // [2][MT*16][GS_ROW]
+    constexpr int ROWS = MT * 16;
+    constexpr int THREADS = 64 * WAVES;
+    constexpr int XCHUNKS = ROWS * (GS_KC / 8) / THREADS;   // 16-byte pieces per thread
+    int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int n0 = blockIdx.x * (16 * WAVES) + wave * 16;
+    int ks = blockIdx.y * k_per_split;
+    int ke = min(k, ks + k_per_split);
+    int n_chunks = (ke - ks + GS_KC - 1) / GS_KC;
+    const bf16_t* wsafe = w + (size_t)min(n0 + (lane & 15), n - 1) * ldw;
+    const bf16_t* wbase = wsafe + (lane >> 4) * 8;
+    u32x4_t w0[8], w1[8], w2[8], xr[XCHUNKS];
+    f32x4_t acc[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        int gm = mt * 16 + (lane & 15);
-        if (gm >= m) continue;
-        if (EPI == EPI_SWIGLU && !PARTIAL) {
-            // a lane holds weight rows 4g .. 4g+3 = two (gate, up) pairs
-#pragma unroll
-            for (int e = 0; e < 4; e += 2) {
-                int gn = n0 + (lane >> 4) * 4 + e;
-                if (gn + 1 < n)
-                    ((bf16_t*)out)[(size_t)gm * ldo + (gn >> 1)] = f32_to_bf16(silu_mul(acc[mt][e], acc[mt][e + 1]));
-            }
-            continue;
-        }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            int gn = n0 + (lane >> 4) * 4 + e;
-            if (gn >= n) continue;
-            if (PARTIAL) ((float*)out)[((size_t)blockIdx.y * m + gm) * n + gn] = acc[mt][e];
-            else epilogue_store<EPI>(out, (size_t)gm * ldo + gn, acc[mt][e]);
-        }
+    for (int i = 0; i < MT; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    // Blocks start their K loop at different chunks and wrap around: row strides are often a
+    // power of two, and blocks that all read the same K window at once would queue up on a few
+    // memory channels.
+    int rot = (blockIdx.x * 5 + blockIdx.y * 3) % n_chunks;
+    // chunk c_ of the loop (clamped to the last one: loads past the end fetch something valid
+    // that nobody uses, so that no load stands under a branch)
+#define GD_CHUNK_BASE(c_) (ks + ((min((c_), n_chunks - 1) + rot) >= n_chunks ? min((c_), n_chunks - 1) + rot - n_chunks : min((c_), n_chunks - 1) + rot) * GS_KC)
+#define GD_LOAD_W(c_, dst_)                                                                     \
+    {                                                                                           \
+        int kb_ = GD_CHUNK_BASE(c_);                                                            \
+        _Pragma("unroll") for (int j = 0; j < 8; ++j) {                                         \
+            bool in_ = kb_ + j * 32 + (lane >> 4) * 8 < ke;                                     \
+            dst_[j] = *(const u32x4_t*)(in_ ? wbase + kb_ + j * 32 : wsafe);                    \
+        }                                                                                       \
     }
+#define GD_LOAD_X(c_)                                                                           \
+    {                                                                                           \
+        int kb_ = GD_CHUNK_BASE(c_);                                                            \
+        _Pragma("unroll") for (int i = 0; i < XCHUNKS; ++i) {                                   \
+            int piece_ = tid + i * THREADS;                                                     \
+            int row_ = piece_ / (GS_KC / 8), gk_ = kb_ + (piece_ % (GS_KC / 8)) * 8;            \
+            xr[i] = *(const u32x4_t*)(gk_ < ke ? x + (size_t)min(row_, m - 1) * ldx + gk_ : x); \
+        }                                                                                       \
+    }
+#define GD_STORE_X(c_, buf_)                                                                    \
+    {                                                                                           \
+        int kb_ = GD_CHUNK_BASE(c_);                                                            \
+        u32x4_t* sx_ = gs_smem + (buf_) * ROWS * GS_ROW;                                        \
+        const u32x4_t zero_ = {0u, 0u, 0u, 0u};                                                 \
+        _Pragma("unroll") for (int i = 0; i < XCHUNKS; ++i) {                                   \
+            int piece_ = tid + i * THREADS;                                                     \
+            int kc_ = piece_ % (GS_KC / 8);                                                     \
+            sx_[(piece_ / (GS_KC / 8)) * GS_ROW + kc_] = kb_ + kc_ * 8 < ke ? xr[i] : zero_;    \
+        }                                                                                       \
+    }
+    // One chunk: the activations of the next chunk and the weights of the chunk after it are
+    // requested (in this order: loads return in order, and the activations are needed first),
+    // the products of this chunk run on weights that were requested two chunks ago, then the
+    // activations go to the other LDS buffer.  Weight loads stay in flight across the barrier:
+    // a wave always has 8 to 16 of them outstanding, which is what keeps the memory busy when
+    // the number of waves is small for the chip.
+    // (neither the optimizer nor the scheduler may move a load across this)
+#define GD_KEEP_ORDER asm volatile("" ::: "memory"); __builtin_amdgcn_sched_barrier(0);
+#define GD_STEP(c_, wcur_, wfar_)                                                               \
+    {                                                                                           \
+        GD_LOAD_X((c_) + 1)                                                                     \
+        GD_KEEP_ORDER                                                                           \
+        GD_LOAD_W((c_) + 2, wfar_)                                                              \
+        GD_KEEP_ORDER                                                                           \
+        const u32x4_t* sx = gs_smem + ((c_) & 1) * ROWS * GS_ROW;                               \
+        _Pragma("unroll") for (int j = 0; j < 8; ++j) {                                         \
+            bf16x8_t a = as_frag4(wcur_[j]);                                                    \
+            _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                 \
+                bf16x8_t b = as_frag4(sx[(mt * 16 + (lane & 15)) * GS_ROW + j * 4 + (lane >> 4)]); \
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);      \
+            }                                                                                   \
+        }                                                                                       \
+        GD_STORE_X((c_) + 1, ((c_) & 1) ^ 1)                                                    \
+        __syncthreads();                                                                        \
+    }
+
+    GD_LOAD_W(0, w0)
+    GD_LOAD_X(0)
+    GD_STORE_X(0, 0)
+    GD_LOAD_W(1, w1)
+    __syncthreads();
+    for (int c = 0; c < n_chunks; c += 3) {
+        GD_STEP(c, w0, w2)
+        if (c + 1 >= n_chunks) break;
+        GD_STEP(c + 1, w1, w0)
+        if (c + 2 >= n_chunks) break;
+        GD_STEP(c + 2, w2, w1)
+    }
+#undef GD_STEP
+#undef GD_KEEP_ORDER
+#undef GD_CHUNK_BASE
+#undef GD_LOAD_W
+#undef GD_LOAD_X
+#undef GD_STORE_X
+    skinny_epilogue<MT, EPI, PARTIAL>(acc, out, ldo, m, n, n0, lane, blockIdx.y);
 }
 
 // ---- at most 16 rows -------------------------------------------------------------------------
