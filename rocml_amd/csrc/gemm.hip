@@ -38,8 +38,8 @@ static int launch_mfma_tile_as(const void* x, int ldx, const void* w, int ldw, v
 }
 
 // shape: 0 = choose, 1 = 128x128 tiles, 2 = 256x256.  Measured in the model (weights from HBM)
-// the big tile reaches about 1030 TFLOP/s on products that fill the chip and the small one
-// about 760 (the wider a wave's own tile and the more waves share an operand, the fewer LDS
+// the big tile reaches about 1060 TFLOP/s on products that fill the chip and the small one
+// about 820 (the wider a wave's own tile and the more waves share an operand, the fewer LDS
 // bytes per product), but a CU holds one big tile or two small ones at a time, and the last
 // round of tiles may leave CUs idle: the choice weighs the speed with the share of the 256 CUs
 // that the rounds keep busy.
@@ -51,7 +51,7 @@ static int launch_mfma_tile(const void* x, int ldx, const void* w, int ldw, void
             double tiles = (double)ceil_div(m, bm) * ceil_div(n, bn);
             return tiles / (ceil_div((long long)tiles, per_round) * (double)per_round);
         };
-        shape = 1030.0 * fill(256, 256, 256) > 760.0 * fill(128, 128, 512) ? 2 : 1;
+        shape = 1060.0 * fill(256, 256, 256) > 820.0 * fill(128, 128, 512) ? 2 : 1;
     }
     if (shape == 2) return launch_mfma_tile_as<EPI, GemmTile256>(x, ldx, w, ldw, out, ldo, m, n, k, stream);
     return launch_mfma_tile_as<EPI, GemmTile128>(x, ldx, w, ldw, out, ldo, m, n, k, stream);

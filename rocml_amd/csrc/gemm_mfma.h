@@ -65,7 +65,11 @@ __device__ __forceinline__ void epilogue_store(void* out, size_t idx, float v) {
 // 64x64 (two blocks per CU) for the rest.  (256x128 with four waves of 128x64 was tried: one
 // wave per SIMD has nobody to cover for it while it waits for weights from HBM.  Reading four
 // bytes of every row's line some stages ahead, to pull it into L2, was tried too: the extra
-// requests cost more than the earlier arrival gains.)
+// requests cost more than the earlier arrival gains.  Loading the operands straight into LDS
+// (global_load_lds_dwordx4, K staged 32 at a time in five unpadded, XOR-swizzled buffers) was
+// tried as well and gave the same results about 7% slower: a barrier every 16 products per wave,
+// and the compiler answers such loads with a full wait on the LDS counter before the first
+// product of every stage.)
 constexpr int GM_BK = 64;
 constexpr int GM_ROW = GM_BK / 8 + 1;                 // u32x4_t per LDS row, one of padding
 
@@ -82,6 +86,30 @@ struct GemmTile {
 using GemmTile128 = GemmTile<2, 2, 2, 2>;
 using GemmTile256 = GemmTile<2, 4, 4, 2>;       // eight waves (two per SIMD), 128x64 each
 
+// Accumulator element e of a lane: row 8*(e/4) + 4*(lane/32) + e%4, column lane%32.
+template <int EPI, typename T>
+__device__ __forceinline__ void tile_epilogue(f32x16_t (&acc)[T::TM][T::TN], void* out, int ldo, int m, int n,
+                                              int m0, int n0, int wm, int wn, int lane) {
+#pragma unroll
+    for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j) {
+            int gn = n0 + (wn * T::TN + j) * 32 + (lane & 31);
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                int gm = m0 + (wm * T::TM + i) * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                if (EPI == EPI_SWIGLU) {
+                    // neighbouring lanes hold neighbouring columns: the even one has the gate
+                    float other = __shfl_xor(acc[i][j][e], 1, 64);
+                    if ((lane & 1) == 0 && gm < m && gn + 1 < n)
+                        ((bf16_t*)out)[(size_t)gm * ldo + (gn >> 1)] = f32_to_bf16(silu_mul(acc[i][j][e], other));
+                } else if (gm < m && gn < n) {
+                    epilogue_store<EPI>(out, (size_t)gm * ldo + gn, acc[i][j][e]);
+                }
+            }
+        }
+}
+
 template <int EPI, typename T>
 __global__ void __launch_bounds__(T::THREADS)
 gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw,
@@ -92,11 +120,12 @@ gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
     constexpr int PROD = T::TM * T::TN;               // products per 16-wide K slice
     constexpr int KK = GM_BK / 16;                    // slices per stage
     static_assert(KK == 4, "the schedule below is written for four slices per stage");
-    // piece r is stored after product r * 2*PROD / NREG of the first two slices; its register is
-    // refilled one product later when every store has a free product behind it, else at the same
-    // place in the last two slices
-    static_assert(2 * PROD >= NREG, "the stores must fit into the first two slices");
-    constexpr bool REFILL_AT_ONCE = 2 * PROD >= 2 * NREG;
+    // piece r is stored after product r * SPAN / NREG of the first three slices (SPAN products);
+    // its register is refilled one product later when every store has a free product behind it,
+    // else right behind the store
+    constexpr int SPAN = 3 * PROD;
+    static_assert(SPAN >= NREG, "the stores must fit into the first three slices");
+    constexpr bool REFILL_LATER = SPAN >= 2 * NREG;
     int per_xcd = gridDim.x / 8;
     int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
     if (logical >= n_tiles) return;
@@ -119,9 +148,10 @@ gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
     //  * the operand pieces of the next slice are read from LDS before the products of the
     //    current slice are issued (two register sets);
     //  * the pieces of the next stage, loaded from global memory one stage ago, are stored to the
-    //    other LDS buffer between the products of slices 0 and 1, and each register is refilled
-    //    from the stage after that: the memory pipes work while the matrix core does, and a load
-    //    has a whole stage to arrive;
+    //    other LDS buffer between the products of slices 0 to 2 (evenly: LDS takes a 128-bit
+    //    store at a quarter of the rate of a read, and bunched stores hold up the operand reads
+    //    behind them), and each register is refilled from the stage after that: the memory pipes
+    //    work while the matrix core does, and a load has a whole stage to arrive;
     //  * the one barrier of a stage stands after slice 2.  By then every wave has stored its
     //    pieces of the next stage and has read the last pieces of this one, so during slice 3 the
     //    first operands of the next stage are fetched and the matrix core does not wait for LDS
@@ -182,17 +212,17 @@ gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
                 acc[q / T::TN][q % T::TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
                     a[c][q / T::TN], b[c][q % T::TN], acc[q / T::TN][q % T::TN], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
-                // the piece whose place is product s of a half stage: r with r * 2*PROD / NREG == s
-                int half_slot = (kk & 1) * PROD + q;
-                int r = (half_slot * NREG + 2 * PROD - 1) / (2 * PROD);
-                bool here = r < NREG && r * 2 * PROD / NREG == half_slot;
-                int rp = ((half_slot - 1) * NREG + 2 * PROD - 1) / (2 * PROD);      // the piece one product earlier
-                bool before = half_slot >= 1 && rp < NREG && rp * 2 * PROD / NREG == half_slot - 1;
-                if (kk < 2) {
-                    if (here) nxt[dst[r]] = in1 ? reg[r] : zero;
-                    else if (REFILL_AT_ONCE && before) reg[rp] = *(const u32x4_t*)(src[rp] + o2);
-                } else if (!REFILL_AT_ONCE && here) {
-                    reg[r] = *(const u32x4_t*)(src[r] + o2);
+                // the piece whose place is product s of the stage: r with r * SPAN / NREG == s
+                int slot = kk * PROD + q;
+                int r = (slot * NREG + SPAN - 1) / SPAN;
+                bool here = kk < 3 && r < NREG && r * SPAN / NREG == slot;
+                int rp = ((slot - 1) * NREG + SPAN - 1) / SPAN;      // the piece one product earlier
+                bool before = slot >= 1 && slot - 1 < SPAN && rp < NREG && rp * SPAN / NREG == slot - 1;
+                if (here) {
+                    nxt[dst[r]] = in1 ? reg[r] : zero;
+                    if (!REFILL_LATER) reg[r] = *(const u32x4_t*)(src[r] + o2);
+                } else if (REFILL_LATER && before) {
+                    reg[rp] = *(const u32x4_t*)(src[rp] + o2);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -200,25 +230,7 @@ gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
         }
     }
 #undef GM_KOFF
-    // Accumulator element e of a lane: row 8*(e/4) + 4*(lane/32) + e%4, column lane%32.
-#pragma unroll
-    for (int i = 0; i < T::TM; ++i)
-#pragma unroll
-        for (int j = 0; j < T::TN; ++j) {
-            int gn = n0 + (wn * T::TN + j) * 32 + (lane & 31);
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                int gm = m0 + (wm * T::TM + i) * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-                if (EPI == EPI_SWIGLU) {
-                    // neighbouring lanes hold neighbouring columns: the even one has the gate
-                    float other = __shfl_xor(acc[i][j][e], 1, 64);
-                    if ((lane & 1) == 0 && gm < m && gn + 1 < n)
-                        ((bf16_t*)out)[(size_t)gm * ldo + (gn >> 1)] = f32_to_bf16(silu_mul(acc[i][j][e], other));
-                } else if (gm < m && gn < n) {
-                    epilogue_store<EPI>(out, (size_t)gm * ldo + gn, acc[i][j][e]);
-                }
-            }
-        }
+    tile_epilogue<EPI, T>(acc, out, ldo, m, n, m0, n0, wm, wn, lane);
 }
 
 // ---- few rows ----------------------------------------------------------------------------
