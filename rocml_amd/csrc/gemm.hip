@@ -21,19 +21,37 @@ static int allow_lds(K kernel, int bytes, const char* name) {
     return 0;
 }
 
+struct SplitPlan { int defer; int* deferred; };
+
 template <int EPI, typename T>
 static int launch_mfma_tile_as(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m,
-                               int n, int k, hipStream_t stream) {
+                               int n, int k, int splits, void* workspace, SplitPlan plan, hipStream_t stream) {
     static bool ready = false;
     if (!ready) {
         if (allow_lds(gemm_mfma_kernel<EPI, T>, T::LDS_BYTES, "gemm")) return 1;
+        if (allow_lds(gemm_mfma_kernel<EPI_F32, T>, T::LDS_BYTES, "gemm")) return 1;
         ready = true;
     }
     int tiles_m = ceil_div(m, T::BM), tiles_n = ceil_div(n, T::BN);
     int n_tiles = tiles_m * tiles_n;
-    int grid = round_up(n_tiles, 8);
-    gemm_mfma_kernel<EPI, T><<<grid, T::THREADS, T::LDS_BYTES, stream>>>(
-        (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, tiles_m, n_tiles);
+    if (splits <= 1) {
+        gemm_mfma_kernel<EPI, T><<<round_up(n_tiles, 8), T::THREADS, T::LDS_BYTES, stream>>>(
+            (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, tiles_m, n_tiles, k, 0);
+        return 0;
+    }
+    // K cut in pieces: 32-bit partial sums [piece][M][N] in the workspace, added in order by the
+    // caller's next kernel or by the reduce kernel here
+    int k_per_split = round_up(ceil_div(k, splits), GM_BK);
+    splits = ceil_div(k, k_per_split);
+    gemm_mfma_kernel<EPI_F32, T><<<round_up(n_tiles * splits, 8), T::THREADS, T::LDS_BYTES, stream>>>(
+        (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, workspace, n, m, n, k, tiles_m, n_tiles, k_per_split,
+        (long long)m * n);
+    if (plan.defer && ldo == n) {
+        *plan.deferred = splits;
+        return 0;
+    }
+    long long total = (long long)m * n;
+    gemm_splitk_reduce_kernel<EPI><<<ceil_div(total, 256), 256, 0, stream>>>((const float*)workspace, out, ldo, m, n, splits);
     return 0;
 }
 
@@ -42,22 +60,28 @@ static int launch_mfma_tile_as(const void* x, int ldx, const void* w, int ldw, v
 // about 820 (the wider a wave's own tile and the more waves share an operand, the fewer LDS
 // bytes per product), but a CU holds one big tile or two small ones at a time, and the last
 // round of tiles may leave CUs idle: the choice weighs the speed with the share of the 256 CUs
-// that the rounds keep busy.
+// that the rounds keep busy.  A product with at most 128 big tiles can have K cut in two, each
+// half the work of a block of its own; the partial sums cost about a tenth of the time.
 template <int EPI>
 static int launch_mfma_tile(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m,
-                            int n, int k, int shape, hipStream_t stream) {
+                            int n, int k, int shape, void* workspace, long long workspace_bytes, SplitPlan plan,
+                            hipStream_t stream) {
+    int splits = 1;
+    auto fill = [&](int bm, int bn, int per_round, int pieces) {
+        double tiles = (double)ceil_div(m, bm) * ceil_div(n, bn) * pieces;
+        return tiles / (ceil_div((long long)tiles, per_round) * (double)per_round);
+    };
+    bool can_split = EPI != EPI_SWIGLU && k >= 2048 && workspace &&
+                     2LL * m * n * (long long)sizeof(float) <= workspace_bytes;
     if (shape == 0) {
-        auto fill = [&](int bm, int bn, int per_round) {
-            double tiles = (double)ceil_div(m, bm) * ceil_div(n, bn);
-            return tiles / (ceil_div((long long)tiles, per_round) * (double)per_round);
-        };
-        shape = 1060.0 * fill(256, 256, 256) > 820.0 * fill(128, 128, 512) ? 2 : 1;
+        double s256 = 1060.0 * fill(256, 256, 256, 1), s256x2 = can_split ? 0.9 * 1060.0 * fill(256, 256, 256, 2) : 0.0,
+               s128 = 820.0 * fill(128, 128, 512, 1);
+        if (s256x2 > s256 && s256x2 > s128) { shape = 2; splits = 2; }
+        else shape = s256 > s128 ? 2 : 1;
     }
-    if (shape == 2) return launch_mfma_tile_as<EPI, GemmTile256>(x, ldx, w, ldw, out, ldo, m, n, k, stream);
-    return launch_mfma_tile_as<EPI, GemmTile128>(x, ldx, w, ldw, out, ldo, m, n, k, stream);
+    if (shape == 2) return launch_mfma_tile_as<EPI, GemmTile256>(x, ldx, w, ldw, out, ldo, m, n, k, splits, workspace, plan, stream);
+    return launch_mfma_tile_as<EPI, GemmTile128>(x, ldx, w, ldw, out, ldo, m, n, k, 1, workspace, plan, stream);
 }
-
-struct SplitPlan { int defer; int* deferred; };
 
 template <int MT, int EPI>
 static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m, int n,
@@ -247,7 +271,8 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
         if (kpar) rc = BY_EPI(launch_kpar, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
         else if (skinny) rc = BY_EPI(launch_skinny_m, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
         else rc = BY_EPI(launch_mfma_tile, x, ldx, w, ldw, out, ldo, m, n, k,
-                         algo == ALGO_MFMA_TILE ? 1 : algo == ALGO_MFMA_TILE256 ? 2 : 0, stream);
+                         algo == ALGO_MFMA_TILE ? 1 : algo == ALGO_MFMA_TILE256 ? 2 : 0, workspace, workspace_bytes,
+                         plan, stream);
 #undef BY_EPI
         if (rc) return rc;
         ROCML_CHECK_LAUNCH("gemm");

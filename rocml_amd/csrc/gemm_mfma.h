@@ -113,7 +113,11 @@ __device__ __forceinline__ void tile_epilogue(f32x16_t (&acc)[T::TM][T::TN], voi
 template <int EPI, typename T>
 __global__ void __launch_bounds__(T::THREADS)
 gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw,
-                 void* __restrict__ out, int ldo, int m, int n, int k, int tiles_m, int n_tiles) {
+                 void* __restrict__ out, int ldo, int m, int n, int k, int tiles_m, int n_tiles,
+                 int k_per_split, long long split_stride) {
+    // With split_stride != 0 the K range is cut into pieces of k_per_split; piece p of a tile is
+    // the work of block p * n_tiles + tile and goes, as 32-bit partial sums, to
+    // out + p * split_stride (the caller instantiates the 32-bit store for that).
     extern __shared__ u32x4_t gm_smem[];              // [2 stages][A: BM rows | B: BN rows][GM_ROW]
     constexpr int STAGE = (T::BM + T::BN) * GM_ROW;
     constexpr int NREG = T::PA + T::PB;               // 16-byte pieces a thread moves per K stage
@@ -128,7 +132,14 @@ gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
     constexpr bool REFILL_LATER = SPAN >= 2 * NREG;
     int per_xcd = gridDim.x / 8;
     int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-    if (logical >= n_tiles) return;
+    int split = logical / n_tiles;
+    logical -= split * n_tiles;
+    int ks = split * k_per_split;
+    if (ks >= k) return;
+    k = min(k - ks, k_per_split);                     // from here on: this block's K range, starting at 0
+    x += ks;
+    w += ks;
+    out = (float*)out + split * split_stride;
     int m0 = (logical % tiles_m) * T::BM, n0 = (logical / tiles_m) * T::BN;
     int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     int wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;

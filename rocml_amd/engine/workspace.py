@@ -17,7 +17,7 @@ import torch
 
 
 class Workspace:
-    def __init__(self, device, scratch_bytes: int = 64 << 20):
+    def __init__(self, device, scratch_bytes: int = 128 << 20):
         self.device = device
         self._buffers: Dict[str, torch.Tensor] = {}
         self.generation = 0

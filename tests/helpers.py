@@ -42,7 +42,15 @@ TINY_E = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "vocab_s
           "rope_theta": 1234.5, "rms_norm_eps": 1e-4, "tie_word_embeddings": False,
           "max_position_embeddings": 300, "hidden_act": "silu", "attention_bias": False}
 
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3), "E": (TINY_E, 4)}
+# Wide enough (K of 2048 and more) for the products of a prompt to be cut along K, with the halves
+# left to the next norm or to the q/k kernel.
+TINY_F = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "vocab_size": 300,
+          "hidden_size": 2048, "intermediate_size": 2112, "num_hidden_layers": 2,
+          "num_attention_heads": 8, "num_key_value_heads": 2, "head_dim": 32,
+          "rope_theta": 10000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True,
+          "max_position_embeddings": 512, "hidden_act": "silu", "attention_bias": False}
+
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3), "E": (TINY_E, 4), "F": (TINY_F, 5)}
 
 
 def make_model_dir(tmp_path, config: Dict, seed: int, dtype=torch.float32) -> str:
