@@ -69,7 +69,7 @@ static int launch_prefill(const AttnArgs& a, hipStream_t stream) {
         if (allow_lds(attn_prefill_mfma_kernel<D>, PrefillLds<D>::BYTES)) return 1;
         ready = true;
     }
-    dim3 grid(a.total_q_tiles, a.hq);
+    dim3 grid(a.total_q_tiles * a.hq);
     attn_prefill_mfma_kernel<D><<<grid, AM_THREADS, PrefillLds<D>::BYTES, stream>>>(
         a.q, a.out, a.kcache, a.vcache, a.block_table, a.bt_width, a.cu_seqlens, a.n_seqs, a.token_pos,
         a.hq, a.hkv, a.scale * LOG2E, a.window);

@@ -204,8 +204,10 @@ __global__ void attn_decode_reduce_kernel(const float* __restrict__ part_o, cons
 }
 
 // ---- prefill: many query tokens per sequence --------------------------------------------------
-// grid (query tiles of 128 rows over all sequences, Hq), 4 waves of 32 query rows.  Pages of
+// grid: query tiles of 128 rows over all sequences x Hq, 4 waves of 32 query rows.  Pages of
 // keys and values go through LDS once per block; every wave multiplies its 32 queries with them.
+constexpr int AM_ROUND = 256;                           // blocks that start together: one per CU
+
 template <int D>
 struct PrefillLds {
     static constexpr int K_ROW = D + 8;                 // bf16 per key row (16 bytes of padding)
@@ -229,10 +231,18 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     bf16_t* sv = sk + AM_PAGE * L::K_ROW;
     int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     int h2 = lane >> 5, col = lane & 31;
-    int h = blockIdx.y, kvh = h / (hq / hkv);
-    // which sequence and which of its query tiles; the last tile of a sequence sees the most
-    // keys, so tiles are handed out from the back: long blocks start first
-    int tile = gridDim.x - 1 - blockIdx.x, b = 0, tok0 = 0, n_new = 0;
+    // Which tile and head.  The last tile of a sequence sees the most keys, the first the fewest.
+    // Blocks are numbered so that (a) heavy tiles come first, all heads of a tile side by side,
+    // and (b) every other round of AM_ROUND blocks runs backwards: the hardware hands block
+    // numbers out in order, a CU that got the r-th heaviest block of a round gets the r-th
+    // lightest of the next, and when all blocks are resident at once (a 2048-token prompt) the
+    // CUs carry equal sums instead of twice the heaviest and twice the lightest.
+    int n_blocks = gridDim.x, total_tiles = n_blocks / hq;
+    int round0 = (blockIdx.x / AM_ROUND) * AM_ROUND, in_round = blockIdx.x - round0;
+    int round_size = min(AM_ROUND, n_blocks - round0);
+    int s = round0 + (((blockIdx.x / AM_ROUND) & 1) ? round_size - 1 - in_round : in_round);
+    int h = s % hq, kvh = h / (hq / hkv);
+    int tile = total_tiles - 1 - s / hq, b = 0, tok0 = 0, n_new = 0;
     for (; b < n_seqs; ++b) {
         tok0 = cu_seqlens[b];
         n_new = cu_seqlens[b + 1] - tok0;
