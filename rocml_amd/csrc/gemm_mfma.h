@@ -65,7 +65,8 @@ __device__ __forceinline__ void epilogue_store(void* out, size_t idx, float v) {
 // 64x64 (two blocks per CU) for the rest.  (256x128 with four waves of 128x64 was tried: one
 // wave per SIMD has nobody to cover for it while it waits for weights from HBM.  Reading four
 // bytes of every row's line some stages ahead, to pull it into L2, was tried too: the extra
-// requests cost more than the earlier arrival gains.  Loading the operands straight into LDS
+// requests cost more than the earlier arrival gains, also when only one block of every tile
+// column (for the weights) and one column in four (for the activations) does it.  Loading the operands straight into LDS
 // (global_load_lds_dwordx4, K staged 32 at a time in five unpadded, XOR-swizzled buffers) was
 // tried as well and gave the same results about 7% slower: a barrier every 16 products per wave,
 // and the compiler answers such loads with a full wait on the LDS counter before the first
