@@ -79,17 +79,32 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         const bf16_t* kbase = kcache + (((size_t)phys * hkv + kvh) * AM_PAGE + half * 32) * D;
         const bf16_t* vbase = vcache + ((size_t)phys * hkv + kvh) * D * AM_PAGE + half * 32;
         int key0 = lpage * AM_PAGE + half * 32;
+        // All loads of the piece go out before anything is computed, the values too: a block has
+        // few pieces, and keys, softmax, values one after the other would be two trips to memory
+        // per piece where one will do.
+        uint4 kreg[2][KD];
+        uint2 va[DT], vb[DT];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const bf16_t* krow = kbase + (size_t)(u * 16 + col) * D + g * 8;
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) kreg[u][kd] = *(const uint4*)(krow + kd * 32);
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const bf16_t* vrow = vbase + (size_t)(dt * 16 + col) * AM_PAGE + g * 4;
+            va[dt] = *(const uint2*)vrow;
+            vb[dt] = *(const uint2*)(vrow + 16);
+        }
+        __builtin_amdgcn_sched_barrier(0);
         // scores of 2 x 16 keys: element i of s[u] is key 16u + 4g + i, column = head.
         f32x4_t s[2];
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             s[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-            const bf16_t* krow = kbase + (size_t)(u * 16 + col) * D + g * 8;
 #pragma unroll
-            for (int kd = 0; kd < KD; ++kd) {
-                bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(krow + kd * 32));
-                s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[kd], s[u], 0, 0, 0);
-            }
+            for (int kd = 0; kd < KD; ++kd)
+                s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kreg[u][kd]), qf[kd], s[u], 0, 0, 0);
         }
         float mx = -INFINITY;
 #pragma unroll
@@ -124,9 +139,7 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         bf16x8_t pf = __builtin_bit_cast(bf16x8_t, pv);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-            const bf16_t* vrow = vbase + (size_t)(dt * 16 + col) * AM_PAGE + g * 4;
-            uint2 a = *(const uint2*)vrow, b = *(const uint2*)(vrow + 16);
-            bf16x8_t vf = __builtin_bit_cast(bf16x8_t, make_uint4(a.x, a.y, b.x, b.y));
+            bf16x8_t vf = __builtin_bit_cast(bf16x8_t, make_uint4(va[dt].x, va[dt].y, vb[dt].x, vb[dt].y));
             o[dt] = o[dt] * corr;
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[dt], 0, 0, 0);
         }
