@@ -96,17 +96,27 @@ __device__ __forceinline__ void tile_epilogue(f32x16_t (&acc)[T::TM][T::TN], voi
 #pragma unroll
         for (int j = 0; j < T::TN; ++j) {
             int gn = n0 + (wn * T::TN + j) * 32 + (lane & 31);
+            if (EPI == EPI_SWIGLU) {
+                // Neighbouring lanes hold neighbouring columns: the even one the gate, the odd one
+                // the up value of one output column.  Of two neighbouring rows the even lane
+                // finishes the first and the odd lane the second: one exchange per pair of rows,
+                // and every lane has half of the exponentials and stores.
+                bool odd = lane & 1;
+#pragma unroll
+                for (int e = 0; e < 16; e += 2) {
+                    float first = acc[i][j][e], second = acc[i][j][e + 1];
+                    float got = __shfl_xor(odd ? first : second, 1, 64);    // even: up of row e; odd: gate of row e+1
+                    float gate = odd ? got : first, up = odd ? second : got;
+                    int gm = m0 + (wm * T::TM + i) * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3) + (odd ? 1 : 0);
+                    if (gm < m && (gn | 1) < n)
+                        ((bf16_t*)out)[(size_t)gm * ldo + (gn >> 1)] = f32_to_bf16(silu_mul(gate, up));
+                }
+                continue;
+            }
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 int gm = m0 + (wm * T::TM + i) * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-                if (EPI == EPI_SWIGLU) {
-                    // neighbouring lanes hold neighbouring columns: the even one has the gate
-                    float other = __shfl_xor(acc[i][j][e], 1, 64);
-                    if ((lane & 1) == 0 && gm < m && gn + 1 < n)
-                        ((bf16_t*)out)[(size_t)gm * ldo + (gn >> 1)] = f32_to_bf16(silu_mul(acc[i][j][e], other));
-                } else if (gm < m && gn < n) {
-                    epilogue_store<EPI>(out, (size_t)gm * ldo + gn, acc[i][j][e]);
-                }
+                if (gm < m && gn < n) epilogue_store<EPI>(out, (size_t)gm * ldo + gn, acc[i][j][e]);
             }
         }
 }
