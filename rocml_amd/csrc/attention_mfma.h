@@ -23,9 +23,7 @@ constexpr int AM_THREADS = 256;
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
-    return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
-}
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) { return f32x2_to_bf16x2(a, b); }
 
 // ---- decode: one query token per sequence ----------------------------------------------------
 // grid (n_splits, Hkv, tokens), 4 waves; the block's pages are cut into 32-key pieces that the

@@ -46,12 +46,16 @@ __device__ __forceinline__ float bf16_to_f32(bf16_t v) {
     return __uint_as_float(((uint32_t)v) << 16);
 }
 
-// Round to nearest even; NaN stays NaN.
-__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (bf16_t)(u >> 16);
+// Round to nearest even; NaN stays NaN.  gfx950 has the conversion in hardware
+// (v_cvt_pk_bf16_f32), which the compiler picks for these casts.
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) { return __builtin_bit_cast(bf16_t, (__bf16)f); }
+
+// two values in one instruction: a in the low half
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(float a, float b) {
+    typedef __attribute__((ext_vector_type(2))) float f32x2_t_;
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t_;
+    f32x2_t_ v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t_));
 }
 
 template <typename T> struct Elem;
