@@ -222,7 +222,7 @@ constexpr int AM_ROUND = 256;                           // blocks that start tog
 template <int D>
 struct PrefillLds {
     static constexpr int K_ROW = D + 8;                 // bf16 per key row (16 bytes of padding)
-    static constexpr int V_ROW = AM_PAGE + 4;           // bf16 per value row (8 bytes of padding)
+    static constexpr int V_ROW = AM_PAGE + 8;           // bf16 per value row (16 bytes of padding)
     static constexpr int BYTES = (AM_PAGE * K_ROW + D * V_ROW) * 2;
 };
 
@@ -325,10 +325,13 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
 #pragma unroll
         for (int i = 0; i < V_PIECES; ++i) {
             int piece = tid + i * AM_THREADS;
+            // Within 16 keys the four groups of 4 stand in the order 0, 2, 1, 3: the second product
+            // wants keys {4h .. 4h+3, 8+4h .. 8+4h+3} per lane (the order the scores come in), and
+            // so finds them side by side, one 16-byte read.
             int d = piece / 8, kc = piece % 8;
-            uint2* dst = (uint2*)(sv + d * L::V_ROW + kc * 8);
+            uint2* dst = (uint2*)(sv + d * L::V_ROW + (kc >> 1) * 16 + (kc & 1) * 4);
             dst[0] = make_uint2(vreg[i][0], vreg[i][1]);
-            dst[1] = make_uint2(vreg[i][2], vreg[i][3]);
+            dst[2] = make_uint2(vreg[i][2], vreg[i][3]);
         }
         __syncthreads();
         if (lpage < last_page) AM_LOAD_PAGE(lpage + 1)
@@ -391,9 +394,8 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
             for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
                 for (int u = 0; u < 2; ++u) {
-                    const bf16_t* vrow = sv + (dt * 32 + col) * L::V_ROW + half * 32 + 16 * u + 4 * h2;
-                    uint2 a = *(const uint2*)vrow, c = *(const uint2*)(vrow + 8);
-                    bf16x8_t vf = __builtin_bit_cast(bf16x8_t, make_uint4(a.x, a.y, c.x, c.y));
+                    const bf16_t* vrow = sv + (dt * 32 + col) * L::V_ROW + half * 32 + 16 * u + 8 * h2;
+                    bf16x8_t vf = __builtin_bit_cast(bf16x8_t, *(const uint4*)vrow);
                     o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[u], o[dt], 0, 0, 0);
                 }
             }
