@@ -25,6 +25,20 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) { return f32x2_to_bf16x2(a, b); }
 
+// Lane l and lane l ^ 32 combined (v_permlane32_swap: one VALU instruction instead of a trip
+// through the LDS crossbar).  After the swap the first word holds the lower half's values in
+// both halves of the wave and the second word the upper half's.
+__device__ __forceinline__ float max_across_halves(float v) {
+    typedef __attribute__((ext_vector_type(2))) unsigned u32x2_;
+    u32x2_ r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_across_halves(float v) {
+    typedef __attribute__((ext_vector_type(2))) unsigned u32x2_;
+    u32x2_ r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // ---- decode: one query token per sequence ----------------------------------------------------
 // grid (n_splits, Hkv, tokens), 4 waves; the block's pages are cut into 32-key pieces that the
 // waves take in turn; all query heads of the kv head ride in the 16 columns of the MFMA.
@@ -336,20 +350,33 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         __syncthreads();
         if (lpage < last_page) AM_LOAD_PAGE(lpage + 1)
         if (!wave_active) continue;
+        // The scores of both 32-key halves are started before either is finished: the softmax of
+        // the first half (vector ALU) then runs while the matrix core still multiplies the second,
+        // and the softmax of the second while the first half's values are multiplied.
+        // S^T: element e of s is key 8(e/4) + 4 h2 + e%4, column = query row.
+        int page_key0 = lpage * AM_PAGE;
+        bool live[2];
+        f32x16_t sc[2];
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
-            int key0 = lpage * AM_PAGE + half * 32;
-            if (key0 > wave_last_key || key0 + 31 < wave_first_key) continue;   // wave-uniform
-            // S^T: element e of s is key 8(e/4) + 4 h2 + e%4, column = query row.
-            f32x16_t s;
+            int key0 = page_key0 + half * 32;
+            live[half] = !(key0 > wave_last_key || key0 + 31 < wave_first_key);   // wave-uniform
+            if (!live[half]) continue;
 #pragma unroll
-            for (int e = 0; e < 16; ++e) s[e] = 0.f;
+            for (int e = 0; e < 16; ++e) sc[half][e] = 0.f;
             const bf16_t* krow = sk + (half * 32 + col) * L::K_ROW + h2 * 8;
 #pragma unroll
             for (int kk = 0; kk < KK; ++kk) {
                 bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(krow + kk * 16));
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], s, 0, 0, 0);
+                sc[half] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], sc[half], 0, 0, 0);
             }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            if (!live[half]) continue;
+            int key0 = page_key0 + half * 32;
+            f32x16_t& s = sc[half];
             bool need_mask = !wave_full || key0 + 31 > wave_min_pos || key0 < wave_max_lo;   // wave-uniform
             if (need_mask) {
 #pragma unroll
@@ -361,7 +388,7 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
             float mx = s[0];
 #pragma unroll
             for (int e = 1; e < 16; ++e) mx = fmaxf(mx, s[e]);
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * scale_log2e;      // the scale is positive
+            mx = max_across_halves(mx) * scale_log2e;       // the scale is positive
             float m_new = fmaxf(m, mx);
             float m_use = m_new == -INFINITY ? 0.f : m_new;
             float sum = 0.f;
@@ -370,7 +397,7 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                 s[e] = fast_exp2(fmaf(s[e], scale_log2e, -m_use));
                 sum += s[e];
             }
-            sum += __shfl_xor(sum, 32, 64);
+            sum = sum_across_halves(sum);
             // the running maximum rarely moves after the first pieces: rescale only when some
             // row of the wave needs it
             if (__builtin_amdgcn_ballot_w64(m_new != m)) {
@@ -391,9 +418,9 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                     pack_bf16x2(s[8 * u + 0], s[8 * u + 1]), pack_bf16x2(s[8 * u + 2], s[8 * u + 3]),
                     pack_bf16x2(s[8 * u + 4], s[8 * u + 5]), pack_bf16x2(s[8 * u + 6], s[8 * u + 7])));
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
+            for (int u = 0; u < 2; ++u) {
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
+                for (int dt = 0; dt < DT; ++dt) {
                     const bf16_t* vrow = sv + (dt * 32 + col) * L::V_ROW + half * 32 + 16 * u + 8 * h2;
                     bf16x8_t vf = __builtin_bit_cast(bf16x8_t, *(const uint4*)vrow);
                     o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[u], o[dt], 0, 0, 0);
