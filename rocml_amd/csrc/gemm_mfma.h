@@ -33,17 +33,7 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;   // 16 bytes as a
 // conditional between two of these is a register select, between two uint4 structs it goes
 // through memory and drags whole arrays into scratch
 
-__device__ __forceinline__ bf16x8_t as_frag(uint4 v) { return __builtin_bit_cast(bf16x8_t, v); }
 __device__ __forceinline__ bf16x8_t as_frag4(u32x4_t v) { return __builtin_bit_cast(bf16x8_t, v); }
-
-// Unconditional 16-byte load from an address the caller has clamped into range, zeroed
-// afterwards when the element is outside the matrix: a load under a branch would be waited for
-// before the next one is issued.
-__device__ __forceinline__ uint4 load16_or_zero(const bf16_t* p, bool ok) {
-    uint4 v = *(const uint4*)p;
-    v.x = ok ? v.x : 0u; v.y = ok ? v.y : 0u; v.z = ok ? v.z : 0u; v.w = ok ? v.w : 0u;
-    return v;
-}
 
 // EPI_SWIGLU: weight rows come in pairs (gate_j, up_j); the output is bfloat16 [M, N/2] with
 // out[m][j] = silu(gate) * up (rocml-kernels/kernels/silu_mul.hip:12-20), formed from the 32-bit
@@ -256,7 +246,7 @@ gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
 }
 
 // ---- few rows ----------------------------------------------------------------------------
-constexpr int GS_BN = 64, GS_KC = 256, GS_THREADS = 256;
+constexpr int GS_KC = 256;                            // K values per chunk
 constexpr int GS_ROW = GS_KC / 8 + 1;                 // uint4 per LDS row of activations
 
 // Accumulator element e of a lane: weight row (lane/16)*4 + e, activation row lane%16.
