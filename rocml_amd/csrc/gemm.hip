@@ -55,32 +55,43 @@ static int launch_mfma_tile_as(const void* x, int ldx, const void* w, int ldw, v
     return 0;
 }
 
-// shape: 0 = choose, 1 = 128x128 tiles, 2 = 256x256.  Measured in the model (weights from HBM)
-// the big tile reaches about 1060 TFLOP/s on products that fill the chip and the small one
-// about 820 (the wider a wave's own tile and the more waves share an operand, the fewer LDS
-// bytes per product), but a CU holds one big tile or two small ones at a time, and the last
-// round of tiles may leave CUs idle: the choice weighs the speed with the share of the 256 CUs
-// that the rounds keep busy.  A product with at most 128 big tiles can have K cut in two, each
-// half the work of a block of its own; the partial sums cost about a tenth of the time.
+// shape: 0 = choose, 1 = 128x128 tiles, 2 = 256x256.  The choice is made on an estimate of the
+// time.  A CU holds one big tile or two small ones; per 64-wide K stage a CU that is kept busy
+// needs about 2.0 us for a big tile and 0.78 us for a small one (measured in the model, weights
+// from HBM: about 1060 and 700 TFLOP/s; the wider a wave's own tile and the more waves share an
+// operand, the fewer LDS bytes per product).  What counts is the CU with the most tiles.  A
+// product with few tiles (few rows, or a narrow output) leaves most CUs idle while a few walk
+// through all of K: then K is cut into up to 8 pieces, each the work of a block of its own,
+// at the price of writing and reading the 32-bit partial sums once more.  No estimate may go
+// below the time the weights need to arrive.
 template <int EPI>
 static int launch_mfma_tile(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m,
                             int n, int k, int shape, void* workspace, long long workspace_bytes, SplitPlan plan,
                             hipStream_t stream) {
     int splits = 1;
-    auto fill = [&](int bm, int bn, int per_round, int pieces) {
-        double tiles = (double)ceil_div(m, bm) * ceil_div(n, bn) * pieces;
-        return tiles / (ceil_div((long long)tiles, per_round) * (double)per_round);
-    };
-    bool can_split = EPI != EPI_SWIGLU && k >= 2048 && workspace &&
-                     2LL * m * n * (long long)sizeof(float) <= workspace_bytes;
     if (shape == 0) {
-        double s256 = 1060.0 * fill(256, 256, 256, 1), s256x2 = can_split ? 0.9 * 1060.0 * fill(256, 256, 256, 2) : 0.0,
-               s128 = 820.0 * fill(128, 128, 512, 1);
-        if (s256x2 > s256 && s256x2 > s128) { shape = 2; splits = 2; }
-        else shape = s256 > s128 ? 2 : 1;
+        double best = 1e30;
+        for (int big = 0; big < 2; ++big) {
+            int edge = big ? 256 : 128;
+            double stage_us = big ? 2.0 : 0.78;
+            long long tiles = (long long)ceil_div(m, edge) * ceil_div(n, edge);
+            for (int pieces = 1; pieces <= 8; ++pieces) {
+                if (pieces > 1 && (EPI == EPI_SWIGLU || k / pieces < 512 || !workspace ||
+                                   (long long)pieces * m * n * (long long)sizeof(float) > workspace_bytes))
+                    break;
+                long long blocks = tiles * pieces;
+                double per_cu = (double)ceil_div(blocks, 256);          // tiles of the busiest CU
+                double stages = (double)ceil_div(ceil_div(k, pieces), GM_BK);
+                double t = per_cu * stages * stage_us + 4.0;
+                if (pieces > 1) t += (double)pieces * m * n * 8.0 / 4.0e6;   // partial sums out and in, 4 TB/s
+                double floor_us = (double)n * k * 2.0 / 5.5e6;               // the weights at 5.5 TB/s
+                if (t < floor_us) t = floor_us;
+                if (t < best) { best = t; shape = big ? 2 : 1; splits = pieces; }
+            }
+        }
     }
     if (shape == 2) return launch_mfma_tile_as<EPI, GemmTile256>(x, ldx, w, ldw, out, ldo, m, n, k, splits, workspace, plan, stream);
-    return launch_mfma_tile_as<EPI, GemmTile128>(x, ldx, w, ldw, out, ldo, m, n, k, 1, workspace, plan, stream);
+    return launch_mfma_tile_as<EPI, GemmTile128>(x, ldx, w, ldw, out, ldo, m, n, k, splits, workspace, plan, stream);
 }
 
 template <int MT, int EPI>
