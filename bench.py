@@ -147,7 +147,8 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b * p_steps / p_dt, 2)
 
     out = {
-        "metric": "decode tok/s (Qwen3-8B shape, bf16, batch 8, 2048-token prompts)",
+        "metric": f"decode tok/s ({args.model} shape, {'bf16' if args.dtype == 'bfloat16' else 'fp32'}, "
+                  f"batch {args.batch}, {PROMPT_LEN}-token prompts)",
         "value": round(value, 2), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
