@@ -1,4 +1,4 @@
-// Sampling on the device, one 256-thread block per sequence, in the order of the reference's
+// Sampling on the device, one 1024-thread block per sequence, in the order of the reference's
 // host sampler (rocml/src/sample.rs:90-166): repeat penalty over recent history, greedy if the
 // temperature is not positive (first maximum wins, :172-182), else scale by 1/temperature,
 // keep the top k, softmax, keep the smallest set of most probable tokens whose mass reaches
@@ -8,6 +8,8 @@
 ROCML_LAST_ERROR_FN(sampling)
 
 constexpr int SB = 256;
+constexpr int SAMPLE_THREADS = 1024;
+constexpr int SAMPLE_MAX_VOCAB = 1 << 20;   // the draw keeps one sum per 256 values in LDS     // the sampling kernel reads a row dozens of times: a big block, 16 bytes per load
 
 struct ArgMax { float v; int i; };
 
@@ -17,6 +19,7 @@ __device__ __forceinline__ ArgMax better(ArgMax a, ArgMax b) {
     return a;
 }
 
+template <int THREADS = SB>
 __device__ ArgMax block_argmax(ArgMax a, ArgMax* scratch) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -30,10 +33,11 @@ __device__ ArgMax block_argmax(ArgMax a, ArgMax* scratch) {
     __syncthreads();
     ArgMax r = scratch[0];
 #pragma unroll
-    for (int w = 1; w < SB / 64; ++w) r = better(r, scratch[w]);
+    for (int w = 1; w < THREADS / 64; ++w) r = better(r, scratch[w]);
     return r;
 }
 
+template <int THREADS = SB>
 __device__ float block_sum_f(float v, float* scratch) {
     v = wave_sum(v);
     __syncthreads();
@@ -41,10 +45,11 @@ __device__ float block_sum_f(float v, float* scratch) {
     __syncthreads();
     float r = 0.f;
 #pragma unroll
-    for (int w = 0; w < SB / 64; ++w) r += scratch[w];
+    for (int w = 0; w < THREADS / 64; ++w) r += scratch[w];
     return r;
 }
 
+template <int THREADS = SB>
 __device__ int block_sum_i(int v, int* scratch) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
@@ -53,9 +58,13 @@ __device__ int block_sum_i(int v, int* scratch) {
     __syncthreads();
     int r = 0;
 #pragma unroll
-    for (int w = 0; w < SB / 64; ++w) r += scratch[w];
+    for (int w = 0; w < THREADS / 64; ++w) r += scratch[w];
     return r;
 }
+
+// e^x for x <= 0 through the hardware's 2^x (v_exp_f32, about one unit in the last place): a
+// sampling call takes the exponential of the whole vocabulary on one CU.
+__device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
 
 // Order-preserving map of a float to an unsigned key (larger float -> larger key).
 __device__ __forceinline__ uint32_t float_key(float f) {
@@ -73,20 +82,134 @@ __device__ __forceinline__ float penalised(float v, int i, const int* hist, int 
     return v;
 }
 
+// The largest of 256 bins whose sum from the top (itself included) reaches `need`, and the sum of
+// the bins above it; bin 0 if the whole histogram falls short.  Called by the 64 lanes of one
+// wave, each with four bins; the sums are integers, so the order of the additions is free.
+template <typename T>
+__device__ __forceinline__ void bin_from_top(const T* bins, T need, int lane, int* bin_out, T* above_out) {
+    T mine = bins[4 * lane] + bins[4 * lane + 1] + bins[4 * lane + 2] + bins[4 * lane + 3];
+    T suffix = mine;                                     // bins of this lane and of all higher lanes
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        T o = __shfl_down(suffix, off, 64);
+        if (lane + off < 64) suffix += o;
+    }
+    unsigned long long reach = __builtin_amdgcn_ballot_w64(suffix >= need);
+    int owner = reach ? 63 - __builtin_clzll(reach) : -1;   // the highest lane from which the top still reaches
+    if (owner < 0) {
+        if (lane == 0) { *bin_out = 0; *above_out = suffix - bins[0]; }
+        return;
+    }
+    if (lane == owner) {
+        T above = suffix - mine;
+        int bin = 4 * lane + 3;
+        for (; bin > 4 * lane; --bin) {
+            if (above + bins[bin] >= need) break;
+            above += bins[bin];
+        }
+        *bin_out = bin;
+        *above_out = above;
+    }
+}
+
+// One pass over a row of `n_` floats by the whole block: BODY sees every index `i_` once with its
+// value `v_`.  Loads go out in batches (four of 16 bytes where the row is aligned, else eight of
+// 4 bytes) before any of them is used: a loop that waits for each load in turn spends its time on
+// latency, and a sampling call makes a dozen passes.  `vec_ok_`: the row starts on 16 bytes.
+#define SAMPLE_ROW_PASS(row_, n_, vec_ok_, i_, v_, ...)                                           \
+    {                                                                                             \
+        int nvec_ = (vec_ok_) ? (n_) / 4 : 0;                                                     \
+        const float4* row4_ = (const float4*)(row_);                                              \
+        for (int base_ = tid; base_ < nvec_; base_ += 4 * SB) {                                   \
+            float4 ld_[4];                                                                        \
+            _Pragma("unroll") for (int u_ = 0; u_ < 4; ++u_) ld_[u_] = row4_[min(base_ + u_ * SB, nvec_ - 1)]; \
+            _Pragma("unroll") for (int u_ = 0; u_ < 4; ++u_) {                                    \
+                if (base_ + u_ * SB < nvec_) {                                                    \
+                    float e_[4] = {ld_[u_].x, ld_[u_].y, ld_[u_].z, ld_[u_].w};                   \
+                    _Pragma("unroll") for (int c_ = 0; c_ < 4; ++c_) {                            \
+                        int i_ = (base_ + u_ * SB) * 4 + c_;                                      \
+                        float v_ = e_[c_];                                                        \
+                        __VA_ARGS__                                                               \
+                    }                                                                             \
+                }                                                                                 \
+            }                                                                                     \
+        }                                                                                         \
+        for (int base_ = nvec_ * 4 + tid; base_ < (n_); base_ += 8 * SB) {                        \
+            float ld_[8];                                                                         \
+            _Pragma("unroll") for (int u_ = 0; u_ < 8; ++u_) ld_[u_] = (row_)[min(base_ + u_ * SB, (n_) - 1)]; \
+            _Pragma("unroll") for (int u_ = 0; u_ < 8; ++u_) {                                    \
+                int i_ = base_ + u_ * SB;                                                         \
+                if (i_ < (n_)) {                                                                  \
+                    float v_ = ld_[u_];                                                           \
+                    __VA_ARGS__                                                                   \
+                }                                                                                 \
+            }                                                                                     \
+        }                                                                                         \
+    }
+
+// The same walk for a pass that rewrites the row: BODY sets `o_` from index `i_` and value `v_`,
+// and the results go out 16 bytes at a time where both rows are aligned (single 4-byte stores of
+// neighbouring lanes land 16 bytes apart and each touches a line of its own).
+#define SAMPLE_ROW_MAP(in_, out_, n_, vec_ok_, i_, v_, o_, ...)                                   \
+    {                                                                                             \
+        int nvec_ = (vec_ok_) ? (n_) / 4 : 0;                                                     \
+        const float4* in4_ = (const float4*)(in_);                                                \
+        float4* out4_ = (float4*)(out_);                                                          \
+        for (int base_ = tid; base_ < nvec_; base_ += 4 * SB) {                                   \
+            float4 ld_[4];                                                                        \
+            _Pragma("unroll") for (int u_ = 0; u_ < 4; ++u_) ld_[u_] = in4_[min(base_ + u_ * SB, nvec_ - 1)]; \
+            _Pragma("unroll") for (int u_ = 0; u_ < 4; ++u_) {                                    \
+                if (base_ + u_ * SB < nvec_) {                                                    \
+                    float e_[4] = {ld_[u_].x, ld_[u_].y, ld_[u_].z, ld_[u_].w};                   \
+                    _Pragma("unroll") for (int c_ = 0; c_ < 4; ++c_) {                            \
+                        int i_ = (base_ + u_ * SB) * 4 + c_;                                      \
+                        float v_ = e_[c_];                                                        \
+                        float o_;                                                                 \
+                        __VA_ARGS__                                                               \
+                        e_[c_] = o_;                                                              \
+                    }                                                                             \
+                    out4_[base_ + u_ * SB] = make_float4(e_[0], e_[1], e_[2], e_[3]);             \
+                }                                                                                 \
+            }                                                                                     \
+        }                                                                                         \
+        for (int base_ = nvec_ * 4 + tid; base_ < (n_); base_ += 8 * SB) {                        \
+            float ld_[8];                                                                         \
+            _Pragma("unroll") for (int u_ = 0; u_ < 8; ++u_) ld_[u_] = (in_)[min(base_ + u_ * SB, (n_) - 1)]; \
+            _Pragma("unroll") for (int u_ = 0; u_ < 8; ++u_) {                                    \
+                int i_ = base_ + u_ * SB;                                                         \
+                if (i_ < (n_)) {                                                                  \
+                    float v_ = ld_[u_];                                                           \
+                    float o_;                                                                     \
+                    __VA_ARGS__                                                                   \
+                    (out_)[i_] = o_;                                                              \
+                }                                                                                 \
+            }                                                                                     \
+        }                                                                                         \
+    }
+
 // logits [B, V] 32-bit.  Per sequence: temperature, top_k (<= 0: off), top_p (<= 0 or >= 1
 // handled as given: off when < 0), u in [0,1), penalty (<= 0: off) with history rows
 // hist[b, 0..hist_len[b]).  work [B, V] 32-bit scratch.  out [B] token ids.
-__global__ void __launch_bounds__(SB)
+__global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_kernel(const float* __restrict__ logits, float* __restrict__ work, int vocab,
               const float* __restrict__ temperature, const int* __restrict__ top_k,
               const float* __restrict__ top_p, const float* __restrict__ uniform,
               const float* __restrict__ penalty, const int* __restrict__ hist, int hist_stride,
               const int* __restrict__ hist_len, int* __restrict__ out) {
+    constexpr int SB = SAMPLE_THREADS;
     __shared__ ArgMax am_scratch[SB / 64];
     __shared__ float f_scratch[SB / 64];
-    __shared__ int i_scratch[SB / 64];
-    __shared__ float seg_sum[SB];
-    __shared__ int seg_cnt[SB];
+    constexpr int WAVES = SB / 64;
+    constexpr int TIE_CAP = 1024, PEN_WORDS = 512, MAX_CHUNKS = SAMPLE_MAX_VOCAB / 256;
+    __shared__ int tie_idx[TIE_CAP];
+    __shared__ int n_ties;
+    __shared__ unsigned pen_bits[PEN_WORDS];
+    __shared__ float chunk_sum[MAX_CHUNKS];
+    __shared__ float seg_base;
+    __shared__ __align__(8) unsigned hist_cnt[WAVES * 256 * 2];   // a histogram per wave: counts, or 64-bit masses
+    __shared__ __align__(8) unsigned bin_cnt[256 * 2];
+    __shared__ int pick[2];
+    __shared__ unsigned long long pick64[2];
     int b = blockIdx.x, tid = threadIdx.x;
     const float* row = logits + (size_t)b * vocab;
     float* wrow = work + (size_t)b * vocab;
@@ -97,16 +220,29 @@ sample_kernel(const float* __restrict__ logits, float* __restrict__ work, int vo
     float temp = temperature[b];
     float inv_temp = temp > 0.f ? 1.0f / temp : 1.0f;
 
-    // pass 1: penalised, scaled logits into work; maximum and its first index.
-    ArgMax best = {-INFINITY, 0x7fffffff};
-    for (int i = tid; i < vocab; i += SB) {
-        float v = row[i];
-        if (nh) v = penalised(v, i, h, nh, pen);
-        ArgMax c = {v, i};
-        best = better(best, c);
-        wrow[i] = v * inv_temp;
+    // pass 1: penalised, scaled logits into work; maximum and its first index.  A token of the
+    // recent history is found through a bitmap over (token mod its size): few tokens pay for the
+    // walk through the history.
+    if (nh) {
+        for (int i = tid; i < PEN_WORDS; i += SB) pen_bits[i] = 0u;
+        __syncthreads();
+        for (int j = tid; j < nh; j += SB) {
+            unsigned t = (unsigned)h[j] % (PEN_WORDS * 32);
+            atomicOr(&pen_bits[t >> 5], 1u << (t & 31));
+        }
+        __syncthreads();
     }
-    best = block_argmax(best, am_scratch);
+    ArgMax best = {-INFINITY, 0x7fffffff};
+    bool row_vec = (uintptr_t)row % 16 == 0, work_vec = (uintptr_t)wrow % 16 == 0;
+    SAMPLE_ROW_MAP(row, wrow, vocab, row_vec && work_vec, i, v, o,
+        if (nh) {
+            unsigned t = (unsigned)i % (PEN_WORDS * 32);
+            if (pen_bits[t >> 5] >> (t & 31) & 1u) v = penalised(v, i, h, nh, pen);
+        }
+        if (v > best.v || best.i == 0x7fffffff) { best.v = v; best.i = i; }   // a thread meets its indices in growing order
+        o = v * inv_temp;
+    )
+    best = block_argmax<SB>(best, am_scratch);
     if (!(temp > 0.f)) {
         if (tid == 0) out[b] = best.i == 0x7fffffff ? 0 : best.i;
         return;
@@ -114,99 +250,232 @@ sample_kernel(const float* __restrict__ logits, float* __restrict__ work, int vo
     float max_logit = best.v * inv_temp;
     __syncthreads();
 
-    // top-k: binary search over the ordered keys for the k-th largest value; candidates are
-    // the values above it plus, among equal ones, the lowest indices up to k.
+    // top-k: the k-th largest value by its ordered key; candidates are the values above it
+    // plus, among equal ones, the lowest indices up to k.
     int k = top_k ? top_k[b] : 0;
     uint32_t kth_key = 0;      // everything is a candidate
     int n_above = 0;
     bool limit_k = k > 0 && k < vocab;
     if (limit_k) {
-        uint32_t lo = 0, hi = 0xffffffffu;   // find largest key T with count(key >= T) >= k
-        while (lo < hi) {
-            uint32_t mid = lo + (uint32_t)(((uint64_t)hi - lo + 1) / 2);
-            int cnt = 0;
-            for (int i = tid; i < vocab; i += SB) cnt += float_key(wrow[i]) >= mid;
-            cnt = block_sum_i(cnt, i_scratch);
-            if (cnt >= k) lo = mid; else hi = mid - 1;
+        // the k-th largest key, 8 bits at a time: a histogram of the next 8 bits over the values
+        // that match the bits found so far, then the bin that holds the k-th from the top
+        uint32_t found = 0;          // leading bits of the k-th key
+        int want = k;                // its rank from the top among the values matching them
+        for (int level = 0; level < 4; ++level) {
+            int shift = 24 - 8 * level;
+            for (int i = tid; i < WAVES * 256; i += SB) hist_cnt[i] = 0;
+            __syncthreads();
+            unsigned* mine = hist_cnt + (tid / 64) * 256;
+            SAMPLE_ROW_PASS(wrow, vocab, work_vec, i, v,
+                uint32_t key = float_key(v);
+                if (level == 0 || (key >> (shift + 8)) == found) atomicAdd(mine + ((key >> shift) & 255), 1u);
+            )
+            __syncthreads();
+            if (tid < 256) {
+                unsigned c = 0;
+                for (int w = 0; w < WAVES; ++w) c += hist_cnt[w * 256 + tid];
+                bin_cnt[tid] = c;
+            }
+            __syncthreads();
+            if (tid < 64) bin_from_top<unsigned>(bin_cnt, (unsigned)want, tid, &pick[0], (unsigned*)&pick[1]);
+            __syncthreads();
+            found = (found << 8) | (uint32_t)pick[0];
+            want -= pick[1];
+            n_above += pick[1];
+            __syncthreads();
         }
-        kth_key = lo;
-        int cnt = 0;
-        for (int i = tid; i < vocab; i += SB) cnt += float_key(wrow[i]) > kth_key;
-        n_above = block_sum_i(cnt, i_scratch);
+        kth_key = found;
     }
     // pass 2: probabilities exp(v - max) of candidates into work, zero elsewhere.  Values equal
-    // to the k-th one are admitted in index order until k candidates are reached: every thread
-    // owns a contiguous segment, counts its ties, and admits those whose rank is below the rest.
-    int per = (vocab + SB - 1) / SB;
-    int s0 = min(vocab, tid * per), s1 = min(vocab, s0 + per);
-    if (limit_k) {
-        int ties_allowed = k - n_above;
-        int mine = 0;
-        for (int i = s0; i < s1; ++i) mine += float_key(wrow[i]) == kth_key;
-        seg_cnt[tid] = mine;
-        __syncthreads();
-        int before = 0;
-        for (int t = 0; t < tid; ++t) before += seg_cnt[t];
-        for (int i = s0; i < s1; ++i) {
-            float v = wrow[i];
+    // to the k-th one are admitted in index order until k candidates are reached: their indices
+    // are collected (there is rarely more than one), ranked among themselves, and the lowest
+    // are written back.
+    if (tid == 0) n_ties = 0;
+    __syncthreads();
+    SAMPLE_ROW_MAP(wrow, wrow, vocab, work_vec, i, v, p,
+        p = fast_exp(v - max_logit);
+        if (limit_k) {
             uint32_t key = float_key(v);
-            bool keep = key > kth_key || (key == kth_key && before++ < ties_allowed);
-            wrow[i] = keep ? expf(v - max_logit) : 0.f;
+            if (key == kth_key) {
+                int slot = atomicAdd(&n_ties, 1);
+                if (slot < TIE_CAP) tie_idx[slot] = i;
+            }
+            if (key <= kth_key) p = 0.f;
         }
-    } else {
-        for (int i = s0; i < s1; ++i) wrow[i] = expf(wrow[i] - max_logit);
-    }
+    )
     __syncthreads();
-    float part = 0.f;
-    for (int i = tid; i < vocab; i += SB) part += wrow[i];
-    float total = block_sum_f(part, f_scratch);
-
-    // top-p: smallest set of the most probable candidates with mass >= p * total.  Binary
-    // search for the largest probability threshold whose mass still reaches it.
-    float p_keep = top_p ? top_p[b] : -1.f;
-    if (p_keep >= 0.f && p_keep < 1.0f) {
-        float target = fminf(fmaxf(p_keep, 0.f), 1.f) * total;
-        uint32_t lo = 0, hi = float_key(1.0f);
-        // largest T with mass(prob >= T) >= target
-        while (lo < hi) {
-            uint32_t mid = lo + (uint32_t)(((uint64_t)hi - lo + 1) / 2);
-            float mass = 0.f;
-            for (int i = tid; i < vocab; i += SB) { float p = wrow[i]; if (p > 0.f && float_key(p) >= mid) mass += p; }
-            mass = block_sum_f(mass, f_scratch);
-            if (mass >= target) lo = mid; else hi = mid - 1;
-        }
-        float kept = 0.f;
-        for (int i = tid; i < vocab; i += SB) {
-            float p = wrow[i];
-            if (!(p > 0.f && float_key(p) >= lo)) { p = 0.f; wrow[i] = 0.f; }
-            kept += p;
-        }
-        __syncthreads();
-        total = block_sum_f(kept, f_scratch);
-    }
-
-    // draw: walk the cumulative mass in index order until it reaches u * total.
-    float threshold = uniform[b] * fmaxf(total, 1.17549435e-38f);
-    float seg = 0.f;
-    for (int i = s0; i < s1; ++i) seg += wrow[i];
-    seg_sum[tid] = seg;
-    __syncthreads();
-    if (tid == 0) {
-        float acc = 0.f;
-        int chosen = -1;
-        for (int t = 0; t < SB && chosen < 0; ++t) {
-            if (acc + seg_sum[t] >= threshold && seg_sum[t] > 0.f) {
-                int a0 = min(vocab, t * per), a1 = min(vocab, a0 + per);
-                for (int i = a0; i < a1; ++i) {
-                    float p = wrow[i];
-                    if (p > 0.f) { acc += p; if (acc >= threshold) { chosen = i; break; } }
-                }
-            } else {
-                acc += seg_sum[t];
+    if (limit_k) {
+        int ties_allowed = k - n_above, ties = n_ties;
+        uint32_t u = (kth_key & 0x80000000u) ? (kth_key & 0x7fffffffu) : ~kth_key;     // the value behind the key
+        float p_tie = fast_exp(__uint_as_float(u) - max_logit);
+        if (ties <= TIE_CAP) {
+            for (int t = tid; t < ties; t += SB) {
+                int mine = tie_idx[t], rank = 0;
+                for (int j = 0; j < ties; ++j) rank += tie_idx[j] < mine;
+                if (rank < ties_allowed) wrow[mine] = p_tie;
+            }
+        } else if (tid == 0) {
+            // a row of thousands of equal values: walk it once, in order
+            int admitted = 0;
+            for (int i = 0; i < vocab && admitted < ties_allowed; ++i) {
+                // the ties are the zeros whose logit has the k-th key; the logits are gone from
+                // the work row, but the input row still has them
+                float v = row[i];
+                if (nh) v = penalised(v, i, h, nh, pen);
+                if (float_key(v * inv_temp) == kth_key) { wrow[i] = p_tie; ++admitted; }
             }
         }
-        if (chosen < 0) chosen = best.i;   // rounding left the threshold above the total
-        out[b] = chosen;
+        __syncthreads();
+    }
+    float part = 0.f;
+    SAMPLE_ROW_PASS(wrow, vocab, work_vec, i, v, part += v; (void)i;)
+    float total = block_sum_f<SB>(part, f_scratch);
+
+    // top-p: smallest set of the most probable candidates with mass >= p * total.
+    float p_keep = top_p ? top_p[b] : -1.f;
+    if (p_keep >= 0.f && p_keep < 1.0f) {
+        // The largest threshold T whose mass(prob >= T) still reaches top_p * total, again 8 bits
+        // of the key at a time.  Masses are added as 40-bit fixed-point integers: the order of
+        // the additions then does not matter and the same row gives the same choice every time.
+        unsigned long long* hist_mass = (unsigned long long*)hist_cnt;      // [WAVES][256] too, twice the bytes
+        unsigned long long* bin_mass = (unsigned long long*)bin_cnt;
+        unsigned long long my_mass = 0ull;
+        SAMPLE_ROW_PASS(wrow, vocab, work_vec, i, p,
+            if (p > 0.f) my_mass += (unsigned long long)(p * 1099511627776.0f);   // p * 2^40, p <= 1
+            (void)i;
+        )
+        for (int off = 32; off > 0; off >>= 1) my_mass += __shfl_xor(my_mass, off, 64);
+        __syncthreads();
+        if ((tid & 63) == 0) bin_mass[tid / 64] = my_mass;
+        __syncthreads();
+        if (tid == 0) {
+            unsigned long long all = 0ull;
+            for (int w = 0; w < WAVES; ++w) all += bin_mass[w];
+            double t = (double)fminf(fmaxf(p_keep, 0.f), 1.f) * (double)all;
+            pick64[0] = t < 1.0 ? 1ull : (unsigned long long)t;     // at least the most probable token
+        }
+        __syncthreads();
+        uint32_t found = 0;
+        for (int level = 0; level < 4; ++level) {
+            int shift = 24 - 8 * level;
+            for (int i = tid; i < WAVES * 256; i += SB) hist_mass[i] = 0ull;
+            __syncthreads();
+            unsigned long long* mine = hist_mass + (tid / 64) * 256;
+            SAMPLE_ROW_PASS(wrow, vocab, work_vec, i, p,
+                uint32_t key = float_key(p);
+                if (p > 0.f && (level == 0 || (key >> (shift + 8)) == found))
+                    atomicAdd(mine + ((key >> shift) & 255u), (unsigned long long)(p * 1099511627776.0f));
+                (void)i;
+            )
+            __syncthreads();
+            if (tid < 256) {
+                unsigned long long c = 0;
+                for (int w = 0; w < WAVES; ++w) c += hist_mass[w * 256 + tid];
+                bin_mass[tid] = c;
+            }
+            __syncthreads();
+            if (tid < 64) bin_from_top<unsigned long long>(bin_mass, pick64[0], tid, &pick[0], &pick64[1]);
+            __syncthreads();
+            if (tid == 0) pick64[0] -= pick64[1];
+            found = (found << 8) | (uint32_t)pick[0];
+            __syncthreads();
+        }
+        uint32_t lo = found;
+        float kept = 0.f;
+        SAMPLE_ROW_MAP(wrow, wrow, vocab, work_vec, i, p, q,
+            q = (p > 0.f && float_key(p) >= lo) ? p : 0.f;
+            kept += q;
+            (void)i;
+        )
+        __syncthreads();
+        total = block_sum_f<SB>(kept, f_scratch);
+    }
+
+    // draw: the first index at which the cumulative mass, in index order, reaches u * total.
+    // The row is cut into chunks of 256 values (4 consecutive ones per lane); every wave adds up
+    // its chunks, one thread walks the chunk sums to the chunk that holds the index, and the
+    // first wave finds the index inside it with a scan over the lanes.
+    float threshold = uniform[b] * fmaxf(total, 1.17549435e-38f);
+    int n_chunks = (vocab + 255) / 256;
+    int lane = tid & 63, wave = tid / 64;
+    for (int c = wave; c < n_chunks; c += WAVES) {
+        int i0 = c * 256 + lane * 4;
+        float sum = 0.f;
+        if (work_vec && i0 + 3 < vocab) {
+            float4 q = *(const float4*)(wrow + i0);
+            sum = ((q.x + q.y) + q.z) + q.w;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sum += i0 + e < vocab ? wrow[i0 + e] : 0.f;
+        }
+        sum = wave_sum(sum);
+        if (lane == 0) chunk_sum[c] = sum;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        // the chunk in which the cumulative mass reaches the threshold: every lane adds up a run
+        // of consecutive chunk sums, a scan over the lanes finds the run, its lane walks it
+        int run = (n_chunks + 63) / 64, c0 = lane * run, c1 = min(n_chunks, c0 + run);
+        float mine = 0.f;
+        for (int c = c0; c < c1; ++c) mine += chunk_sum[c];
+        float upto = mine;                                   // inclusive scan over the lanes
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            float o = __shfl_up(upto, off, 64);
+            if (lane >= off) upto += o;
+        }
+        unsigned long long reach = __builtin_amdgcn_ballot_w64(mine > 0.f && upto >= threshold);
+        int owner = reach ? __builtin_ctzll(reach) : -1;     // the first lane whose run reaches it
+        if (owner < 0 && lane == 0) pick[0] = n_chunks;
+        if (lane == owner) {
+            float acc = upto - mine;
+            int c = c0;
+            for (; c < c1; ++c) {
+                if (chunk_sum[c] > 0.f && acc + chunk_sum[c] >= threshold) break;
+                acc += chunk_sum[c];
+            }
+            if (c == c1) {                                   // rounding inside the run: its last chunk with mass
+                for (c = c1 - 1; c > c0 && !(chunk_sum[c] > 0.f); --c) {}
+                acc = upto - mine;
+                for (int j = c0; j < c; ++j) acc += chunk_sum[j];
+            }
+            pick[0] = c;
+            seg_base = acc;
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {
+        int c = pick[0], chosen = 0x7fffffff, last_positive = -1;
+        if (c < n_chunks) {
+            int i0 = c * 256 + lane * 4;
+            float v[4], mine = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { v[e] = i0 + e < vocab ? wrow[i0 + e] : 0.f; mine += v[e]; }
+            float before = mine;                                // inclusive scan over the lanes
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                float o = __shfl_up(before, off, 64);
+                if (lane >= off) before += o;
+            }
+            float acc = seg_base + (before - mine);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (v[e] > 0.f) {
+                    acc += v[e];
+                    last_positive = i0 + e;
+                    if (acc >= threshold && chosen == 0x7fffffff) chosen = i0 + e;
+                }
+            }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            chosen = min(chosen, __shfl_xor(chosen, off, 64));
+            last_positive = max(last_positive, __shfl_xor(last_positive, off, 64));
+        }
+        // the chunk's sum was added up in another order than the scan: if rounding leaves the scan
+        // short of the threshold, the chunk's last candidate is meant; without any chunk (the
+        // threshold above the total by rounding) the most probable token
+        if (lane == 0) out[b] = chosen != 0x7fffffff ? chosen : (last_positive >= 0 ? last_positive : best.i);
     }
 }
 
@@ -216,8 +485,9 @@ ROCML_EXPORT int rocml_sample(const float* logits, float* work, int batch, int v
                               int hist_stride, const int* hist_len, int* out, hipStream_t stream) {
     ROCML_REQUIRE(batch >= 0 && vocab > 0, "sample: bad sizes B=%d V=%d", batch, vocab);
     ROCML_REQUIRE(logits && work && temperature && uniform && out, "sample: null argument");
+    ROCML_REQUIRE(vocab <= SAMPLE_MAX_VOCAB, "sample: vocabulary %d exceeds %d", vocab, SAMPLE_MAX_VOCAB);
     if (batch == 0) return 0;
-    sample_kernel<<<batch, SB, 0, stream>>>(logits, work, vocab, temperature, top_k, top_p, uniform,
+    sample_kernel<<<batch, SAMPLE_THREADS, 0, stream>>>(logits, work, vocab, temperature, top_k, top_p, uniform,
                                             penalty, hist, hist_stride, hist_len, out);
     ROCML_CHECK_LAUNCH("sample");
     return 0;
