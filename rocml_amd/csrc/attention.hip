@@ -58,7 +58,8 @@ static int launch_decode(const AttnArgs& a, hipStream_t stream) {
         a.q, a.out, a.kcache, a.vcache, a.block_table, a.bt_width, a.token_seq, a.token_pos, a.hq, a.hkv,
         a.scale * LOG2E, a.window, n_splits, part_o, part_ml);
     if (n_splits > 1)
-        attn_decode_reduce_kernel<D><<<a.n_tokens * a.hq, D < 64 ? 64 : D, 0, stream>>>(part_o, part_ml, a.out, n_splits);
+        // whole waves: the kernel's reductions exchange values between all 64 lanes
+        attn_decode_reduce_kernel<D><<<a.n_tokens * a.hq, (D + 63) / 64 * 64, 0, stream>>>(part_o, part_ml, a.out, n_splits);
     return 0;
 }
 

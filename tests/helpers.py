@@ -50,7 +50,16 @@ TINY_F = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "vocab_s
           "rope_theta": 10000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True,
           "max_position_embeddings": 512, "hidden_act": "silu", "attention_bias": False}
 
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3), "E": (TINY_E, 4), "F": (TINY_F, 5)}
+# A head size of 96 (one and a half waves wide where a kernel takes a thread per value) with
+# eight query heads on each key/value head, three layers.
+TINY_G = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "vocab_size": 1000,
+          "hidden_size": 128, "intermediate_size": 176, "num_hidden_layers": 3,
+          "num_attention_heads": 16, "num_key_value_heads": 2, "head_dim": 96,
+          "rope_theta": 10000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": False,
+          "max_position_embeddings": 512, "hidden_act": "silu", "attention_bias": False}
+
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3), "E": (TINY_E, 4), "F": (TINY_F, 5),
+        "G": (TINY_G, 22)}
 
 
 def make_model_dir(tmp_path, config: Dict, seed: int, dtype=torch.float32) -> str:

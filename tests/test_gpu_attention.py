@@ -97,7 +97,7 @@ def _check(seqs, hq, hkv, d, dtype, algo, window=None, n_splits=0, seed=0):
 DECODE = [(16, 8, 128, 1, 0), (16, 8, 128, 3, 0), (16, 8, 128, 33, 0), (16, 8, 128, 257, 1), (16, 8, 128, 257, 4),
           (16, 8, 128, 2048, 1), (16, 8, 128, 2048, 8), (8, 2, 256, 400, 0), (8, 2, 256, 1024, 6),
           (8, 8, 128, 300, 0), (16, 8, 128, 100, 0), (6, 2, 32, 77, 3), (4, 1, 64, 130, 2), (16, 1, 64, 65, 0),
-          (12, 4, 96, 200, 0)]
+          (12, 4, 96, 200, 0), (12, 4, 96, 200, 3), (16, 2, 96, 9, 2), (24, 3, 192, 500, 5)]
 
 
 @pytest.mark.parametrize("hq,hkv,d,length,splits", DECODE)
