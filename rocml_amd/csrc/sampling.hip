@@ -66,9 +66,11 @@ __device__ int block_sum_i(int v, int* scratch) {
 // sampling call takes the exponential of the whole vocabulary on one CU.
 __device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
 
-// Order-preserving map of a float to an unsigned key (larger float -> larger key).
+// Order-preserving map of a float to an unsigned key (larger float -> larger key).  The two
+// zeros compare equal as numbers and so share one key: a tie between them goes by token id.
 __device__ __forceinline__ uint32_t float_key(float f) {
     uint32_t u = __float_as_uint(f);
+    if (u == 0x80000000u) u = 0;
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 

@@ -117,6 +117,20 @@ def test_ties_at_the_kth_value_keep_the_lowest_ids():
     assert got == {10, 50}
 
 
+def test_the_two_zeros_tie():
+    """-0.0 and +0.0 are one value: among them the lowest ids are kept, whatever their signs."""
+    logits = torch.full((1, 200), -3.0)
+    zeros = [4, 9, 20, 33, 61, 150]
+    logits[0, zeros] = torch.tensor([-0.0, 0.0, -0.0, 0.0, 0.0, -0.0])
+    got = set(_draw(logits.expand(32, 200).contiguous(), [SamplingParams(temperature=1.3, top_k=3)] * 32,
+                    [(i + 0.5) / 32 for i in range(32)]))
+    assert got == {4, 9, 20}
+    logits[logits < -1] = -30.0
+    got = set(_draw(logits.expand(32, 200).contiguous(), [SamplingParams(temperature=1.3, top_k=50, top_p=0.5)] * 32,
+                    [(i + 0.5) / 32 for i in range(32)]))
+    assert got == set(zeros)                                # ties with the nucleus' last value stay
+
+
 def test_penalty_changes_the_greedy_choice():
     logits = torch.zeros(1, 50)
     logits[0, 7], logits[0, 9] = 3.0, 2.9
