@@ -86,30 +86,32 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     for (int i = 0; i < DT; ++i) o[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     for (int piece = wave; piece < n_pieces; piece += 4) {
-        int lpage = p_begin + (piece >> 1), half = piece & 1;
+        // (the page index is the same for all lanes: a scalar load)
+        int lpage = __builtin_amdgcn_readfirstlane(p_begin + (piece >> 1)), half = piece & 1;
         int phys = pages[lpage];
         const bf16_t* kbase = kcache + (((size_t)phys * hkv + kvh) * AM_PAGE + half * 32) * D;
         const bf16_t* vbase = vcache + ((size_t)phys * hkv + kvh) * D * AM_PAGE + half * 32;
         int key0 = lpage * AM_PAGE + half * 32;
         // All loads of the piece go out before anything is computed, the values too: a block has
         // few pieces, and keys, softmax, values one after the other would be two trips to memory
-        // per piece where one will do.
-        uint4 kreg[2][KD];
-        uint2 va[DT], vb[DT];
+        // per piece where one will do.  (Requesting the next piece while this one is multiplied
+        // was tried: with eight waves per CU the memory is busy anyway, and short sequences paid
+        // for the extra request at their end.)
+        // Row r of score tile u is key 8 (r / 4) + 4u + r % 4 of the piece: then the 8 keys whose
+        // probabilities a lane holds after the softmax (rows 4g .. 4g+3 of both tiles) are the
+        // consecutive keys 8g .. 8g+7, and its values for them are one 16-byte load.
+        uint4 kreg[2][KD], vreg[DT];
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            const bf16_t* krow = kbase + (size_t)(u * 16 + col) * D + g * 8;
+            const bf16_t* krow = kbase + (size_t)(8 * (col >> 2) + 4 * u + (col & 3)) * D + g * 8;
 #pragma unroll
             for (int kd = 0; kd < KD; ++kd) kreg[u][kd] = *(const uint4*)(krow + kd * 32);
         }
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            const bf16_t* vrow = vbase + (size_t)(dt * 16 + col) * AM_PAGE + g * 4;
-            va[dt] = *(const uint2*)vrow;
-            vb[dt] = *(const uint2*)(vrow + 16);
-        }
+        for (int dt = 0; dt < DT; ++dt)
+            vreg[dt] = *(const uint4*)(vbase + (size_t)(dt * 16 + col) * AM_PAGE + g * 8);
         __builtin_amdgcn_sched_barrier(0);
-        // scores of 2 x 16 keys: element i of s[u] is key 16u + 4g + i, column = head.
+        // scores of 2 x 16 keys: element i of s[u] is key 8g + 4u + i, column = head.
         f32x4_t s[2];
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
@@ -123,7 +125,7 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         for (int u = 0; u < 2; ++u)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                int key = key0 + u * 16 + g * 4 + i;
+                int key = key0 + g * 8 + u * 4 + i;
                 float v = (key >= lo && key < len) ? s[u][i] * scale_log2e : -INFINITY;
                 s[u][i] = v;
                 mx = fmaxf(mx, v);
@@ -145,15 +147,14 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         sum += __shfl_xor(sum, 32, 64);
         l = l * corr + sum;
         m = m_new;
-        // P^T operand: slots 0..3 = keys 4g..4g+3, slots 4..7 = keys 16+4g..16+4g+3.
+        // P^T operand: slots 0..7 = keys 8g .. 8g+7.
         uint4 pv = make_uint4(pack_bf16x2(s[0][0], s[0][1]), pack_bf16x2(s[0][2], s[0][3]),
                               pack_bf16x2(s[1][0], s[1][1]), pack_bf16x2(s[1][2], s[1][3]));
         bf16x8_t pf = __builtin_bit_cast(bf16x8_t, pv);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-            bf16x8_t vf = __builtin_bit_cast(bf16x8_t, make_uint4(va[dt].x, va[dt].y, vb[dt].x, vb[dt].y));
             o[dt] = o[dt] * corr;
-            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[dt], 0, 0, 0);
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vreg[dt]), pf, o[dt], 0, 0, 0);
         }
     }
     // merge the four waves in wave order; element i of o[dt] is d = 16 dt + 4g + i, column = head.
