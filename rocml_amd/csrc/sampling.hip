@@ -8,8 +8,8 @@
 ROCML_LAST_ERROR_FN(sampling)
 
 constexpr int SB = 256;
-constexpr int SAMPLE_THREADS = 1024;
-constexpr int SAMPLE_MAX_VOCAB = 1 << 20;   // the draw keeps one sum per 256 values in LDS     // the sampling kernel reads a row dozens of times: a big block, 16 bytes per load
+constexpr int SAMPLE_THREADS = 1024;        // the sampling kernel reads a row dozens of times: a big block, 16 bytes per load
+constexpr int SAMPLE_MAX_VOCAB = 1 << 20;   // the draw keeps one sum per 256 values in LDS
 
 struct ArgMax { float v; int i; };
 
@@ -202,10 +202,11 @@ sample_kernel(const float* __restrict__ logits, float* __restrict__ work, int vo
     __shared__ ArgMax am_scratch[SB / 64];
     __shared__ float f_scratch[SB / 64];
     constexpr int WAVES = SB / 64;
-    constexpr int TIE_CAP = 1024, PEN_WORDS = 512, MAX_CHUNKS = SAMPLE_MAX_VOCAB / 256;
+    constexpr int TIE_CAP = 1024, PEN_WORDS = 2048, PEN_HIST = 256, MAX_CHUNKS = SAMPLE_MAX_VOCAB / 256;
     __shared__ int tie_idx[TIE_CAP];
     __shared__ int n_ties;
     __shared__ unsigned pen_bits[PEN_WORDS];
+    __shared__ int pen_hist[PEN_HIST];                 // the history, when it fits: a token that pays for the walk pays LDS reads, not trips to memory
     __shared__ float chunk_sum[MAX_CHUNKS];
     __shared__ float seg_base;
     __shared__ __align__(8) unsigned hist_cnt[WAVES * 256 * 2];   // a histogram per wave: counts, or 64-bit masses
@@ -223,27 +224,48 @@ sample_kernel(const float* __restrict__ logits, float* __restrict__ work, int vo
     float inv_temp = temp > 0.f ? 1.0f / temp : 1.0f;
 
     // pass 1: penalised, scaled logits into work; maximum and its first index.  A token of the
-    // recent history is found through a bitmap over (token mod its size): few tokens pay for the
-    // walk through the history.
+    // recent history is found through a bitmap over (token mod its size); the few tokens that
+    // the bitmap flags are set aside (in the list that later holds the ties) and walk through the
+    // history after the pass, a thread each: a walk inside the pass would stand between its
+    // batched loads and their use.
     if (nh) {
         for (int i = tid; i < PEN_WORDS; i += SB) pen_bits[i] = 0u;
+        if (tid == 0) n_ties = 0;
         __syncthreads();
         for (int j = tid; j < nh; j += SB) {
-            unsigned t = (unsigned)h[j] % (PEN_WORDS * 32);
+            int tok = h[j];
+            if (j < PEN_HIST) pen_hist[j] = tok;
+            unsigned t = (unsigned)tok % (PEN_WORDS * 32);
             atomicOr(&pen_bits[t >> 5], 1u << (t & 31));
         }
         __syncthreads();
+        if (nh <= PEN_HIST) h = pen_hist;
     }
     ArgMax best = {-INFINITY, 0x7fffffff};
     bool row_vec = (uintptr_t)row % 16 == 0, work_vec = (uintptr_t)wrow % 16 == 0;
     SAMPLE_ROW_MAP(row, wrow, vocab, row_vec && work_vec, i, v, o,
+        bool later = false;
         if (nh) {
             unsigned t = (unsigned)i % (PEN_WORDS * 32);
-            if (pen_bits[t >> 5] >> (t & 31) & 1u) v = penalised(v, i, h, nh, pen);
+            if (pen_bits[t >> 5] >> (t & 31) & 1u) {
+                int slot = atomicAdd(&n_ties, 1);
+                if (slot < TIE_CAP) { tie_idx[slot] = i; later = true; }
+                else v = penalised(v, i, h, nh, pen);                           // the list is full: walk here
+            }
         }
-        if (v > best.v || best.i == 0x7fffffff) { best.v = v; best.i = i; }   // a thread meets its indices in growing order
+        if (!later && (v > best.v || best.i == 0x7fffffff)) { best.v = v; best.i = i; }   // a thread meets its indices in growing order
         o = v * inv_temp;
     )
+    if (nh) {
+        __syncthreads();
+        int n_later = min(n_ties, TIE_CAP);
+        for (int r = tid; r < n_later; r += SB) {
+            int i = tie_idx[r];
+            ArgMax mine = {penalised(row[i], i, h, nh, pen), i};
+            wrow[i] = mine.v * inv_temp;
+            best = better(best, mine);
+        }
+    }
     best = block_argmax<SB>(best, am_scratch);
     if (!(temp > 0.f)) {
         if (tid == 0) out[b] = best.i == 0x7fffffff ? 0 : best.i;

@@ -139,6 +139,25 @@ def test_penalty_changes_the_greedy_choice():
     assert _draw(logits, [SamplingParams(repeat_penalty=1.0)], [0.0], [[7]]) == [7]
 
 
+def test_penalty_with_a_long_history_in_a_large_vocabulary():
+    """More flagged tokens than the kernel sets aside for later, and a history longer than its
+    copy in LDS: the penalised maximum and the draws must still be the plain rule's."""
+    g = torch.Generator().manual_seed(5)
+    vocab, window = 700001, 600
+    logits = torch.randn(2, vocab, generator=g) * 2.0
+    top = [int(t) for t in logits[0].topk(300).indices]           # the best tokens are all penalised
+    history = top + [int(t) for t in torch.randint(0, vocab, (300,), generator=g)]
+    greedy = SamplingParams(repeat_penalty=1.7, repeat_penalty_window=window)
+    want = [int(np.argmax(np.where(candidates(logits[r].numpy(), 0.0, None, None, 1.7, history, window) > 0, 1, 0)))
+            for r in range(2)]
+    assert _draw(logits, [greedy] * 2, [0.0] * 2, [history] * 2) == want
+    assert want[0] not in top[:50]
+    draw = SamplingParams(temperature=0.8, top_k=40, repeat_penalty=1.7, repeat_penalty_window=window)
+    p = candidates(logits[0].numpy(), 0.8, 40, None, 1.7, history, window)
+    got = _draw(logits[:1].expand(16, vocab).contiguous(), [draw] * 16, [(i + 0.5) / 16 for i in range(16)], [history] * 16)
+    assert all(p[t] > 0 for t in got) and len(set(got)) > 4
+
+
 def test_same_seed_same_draws_and_own_stream_per_sequence():
     g = torch.Generator().manual_seed(3)
     logits = torch.randn(3, 700, generator=g)
