@@ -503,14 +503,197 @@ sample_kernel(const float* __restrict__ logits, float* __restrict__ work, int vo
     }
 }
 
+// ---- a small top-k: slices, then one wave ------------------------------------------------------
+// With a top-k of at most SMALL_K everything after the selection concerns k candidates, and the
+// selection splits: the vocabulary is cut into at most 64 slices, a block per slice and sequence
+// keeps its slice in registers (penalty and temperature applied) and hands out its k best in
+// order (value descending, then index ascending: the order in which ties are admitted); the k
+// best of the row are among these.  One wave per sequence then merges the sorted lists, a lane
+// per slice, and lane r ends up with the r-th best: softmax, top-p and the draw are a matter of
+// shuffles.  The rules are those of sample_kernel above; a row is read once, by many CUs,
+// instead of a dozen times by one.
+constexpr int SMALL_K = 64, SLICE_THREADS = 256, MAX_SLICES = 64;
+
+template <int EPT>
+__global__ void __launch_bounds__(SLICE_THREADS)
+sample_slice_topk_kernel(const float* __restrict__ logits, int vocab, int slice_len,
+                         const float* __restrict__ temperature, const int* __restrict__ top_k,
+                         const float* __restrict__ penalty, const int* __restrict__ hist, int hist_stride,
+                         const int* __restrict__ hist_len, int k_stride, float* __restrict__ cand_v,
+                         int* __restrict__ cand_i) {
+    __shared__ ArgMax am_scratch[SLICE_THREADS / 64];
+    int s = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    int base = s * slice_len, end = min(vocab, base + slice_len);
+    float temp = temperature[b];
+    bool greedy = !(temp > 0.f);
+    float inv_temp = greedy ? 1.0f : 1.0f / temp;
+    int k = greedy ? 1 : min(max(top_k[b], 1), k_stride);
+    const float* row = logits + (size_t)b * vocab;
+    float v[EPT];
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+        int i = base + e * SLICE_THREADS + tid;
+        v[e] = i < end ? row[i] : -INFINITY;
+    }
+    float pen = penalty ? penalty[b] : 0.f;
+    if (pen > 0.f && fabsf(pen - 1.0f) >= 1.1920929e-07f && hist && hist_len) {
+        // once per occurrence in the history, as the reference does; the thread that holds the
+        // token applies it
+        const int* h = hist + (size_t)b * hist_stride;
+        int nh = hist_len[b];
+        for (int j = 0; j < nh; ++j) {
+            int off = h[j] - base;
+            if (off >= 0 && off < end - base && off % SLICE_THREADS == tid) {
+                int we = off / SLICE_THREADS;
+#pragma unroll
+                for (int e = 0; e < EPT; ++e)
+                    if (e == we) v[e] = v[e] > 0.f ? v[e] / pen : v[e] * pen;
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) v[e] *= inv_temp;     // (-inf stays -inf)
+    float* out_v = cand_v + ((size_t)b * gridDim.x + s) * k_stride;
+    int* out_i = cand_i + ((size_t)b * gridDim.x + s) * k_stride;
+    for (int r = 0; r < k; ++r) {
+        // a thread's indices grow with e: its first maximum is its lowest index
+        ArgMax mine = {-INFINITY, 0x7fffffff};
+#pragma unroll
+        for (int e = 0; e < EPT; ++e)
+            if (v[e] > mine.v) { mine.v = v[e]; mine.i = base + e * SLICE_THREADS + tid; }
+        ArgMax win = block_argmax<SLICE_THREADS>(mine, am_scratch);
+        if (tid == 0) { out_v[r] = win.v; out_i[r] = win.i; }
+        if (win.i == 0x7fffffff) {                      // the slice is used up: the rest of the list is empty
+            for (int q = r + 1 + tid; q < k; q += SLICE_THREADS) { out_v[q] = -INFINITY; out_i[q] = 0x7fffffff; }
+            break;
+        }
+        if ((win.i - base) % SLICE_THREADS == tid) {
+            int we = (win.i - base) / SLICE_THREADS;
+#pragma unroll
+            for (int e = 0; e < EPT; ++e)
+                if (e == we) v[e] = -INFINITY;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(64)
+sample_merge_draw_kernel(const float* __restrict__ cand_v, const int* __restrict__ cand_i, int n_slices,
+                         int k_stride, const float* __restrict__ temperature, const int* __restrict__ top_k,
+                         const float* __restrict__ top_p, const float* __restrict__ uniform,
+                         int* __restrict__ out) {
+    __shared__ float sv[MAX_SLICES * SMALL_K];
+    __shared__ int si[MAX_SLICES * SMALL_K];
+    int b = blockIdx.x, lane = threadIdx.x;
+    float temp = temperature[b];
+    bool greedy = !(temp > 0.f);
+    int k = greedy ? 1 : min(max(top_k[b], 1), k_stride);
+    for (int idx = lane; idx < n_slices * k; idx += 64) {
+        int s = idx / k, r = idx - s * k;
+        sv[s * SMALL_K + r] = cand_v[((size_t)b * n_slices + s) * k_stride + r];
+        si[s * SMALL_K + r] = cand_i[((size_t)b * n_slices + s) * k_stride + r];
+    }
+    __syncthreads();
+    // merge of the sorted lists, a lane per slice: lane r keeps the r-th best of the row
+    int ptr = 0;
+    ArgMax mine = {-INFINITY, 0x7fffffff};
+    for (int r = 0; r < k; ++r) {
+        ArgMax head = {-INFINITY, 0x7fffffff};
+        if (lane < n_slices && ptr < k) { head.v = sv[lane * SMALL_K + ptr]; head.i = si[lane * SMALL_K + ptr]; }
+        ArgMax win = head;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            ArgMax o;
+            o.v = __shfl_xor(win.v, off, 64);
+            o.i = __shfl_xor(win.i, off, 64);
+            win = better(win, o);
+        }
+        if (win.i != 0x7fffffff && head.i == win.i) ++ptr;
+        if (lane == r) mine = win;
+    }
+    if (greedy) {
+        if (lane == 0) out[b] = mine.i == 0x7fffffff ? 0 : mine.i;
+        return;
+    }
+    bool valid = lane < k && mine.i != 0x7fffffff;
+    float top_v = __shfl(mine.v, 0, 64);
+    float p = valid ? fast_exp(mine.v - top_v) : 0.f;
+    // top-p over the candidates in descending order: the shortest prefix whose mass reaches
+    // top_p of the total, and every candidate as probable as its last one
+    bool keep = valid;
+    float tp = top_p ? top_p[b] : -1.0f;
+    if (tp >= 0.f && tp < 1.0f) {
+        double cum = (double)p;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            double o = __shfl_up(cum, off, 64);
+            if (lane >= off) cum += o;
+        }
+        double total = __shfl(cum, 63, 64);
+        unsigned long long reached = __builtin_amdgcn_ballot_w64(valid && cum >= (double)tp * total);
+        unsigned long long any = __builtin_amdgcn_ballot_w64(valid);
+        int cut = reached ? __builtin_ctzll(reached) : (any ? 63 - __builtin_clzll(any) : 0);
+        float last_p = __shfl(p, cut, 64);
+        keep = valid && p >= last_p;
+    }
+    // the draw walks the kept candidates in index order
+    double below = 0.0, total_kept = 0.0;
+    for (int j = 0; j < k; ++j) {
+        float pj = __shfl(p, j, 64);
+        int ij = __shfl(mine.i, j, 64);
+        bool kj = __shfl((int)keep, j, 64) != 0;
+        if (kj) {
+            total_kept += (double)pj;
+            if (ij < mine.i) below += (double)pj;
+        }
+    }
+    double t = (double)uniform[b] * total_kept;
+    unsigned long long hit = __builtin_amdgcn_ballot_w64(keep && below <= t && t < below + (double)p);
+    // (a threshold at or above the total by rounding means the last kept candidate in index order)
+    int chosen;
+    if (hit) {
+        chosen = __shfl(mine.i, __builtin_ctzll(hit), 64);
+    } else {
+        int cand = keep ? mine.i : -1;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) cand = max(cand, __shfl_xor(cand, off, 64));
+        chosen = cand >= 0 ? cand : (__shfl(mine.i, 0, 64) == 0x7fffffff ? 0 : __shfl(mine.i, 0, 64));
+    }
+    if (lane == 0) out[b] = chosen;
+}
+
+// small_k: 0, or a bound (at most SMALL_K) that every sequence's top_k lies in [1, small_k] under
+// (sequences with a temperature <= 0 aside): then the slice kernels run, if the workspace holds
+// their candidate lists.
 ROCML_EXPORT int rocml_sample(const float* logits, float* work, int batch, int vocab,
                               const float* temperature, const int* top_k, const float* top_p,
                               const float* uniform, const float* penalty, const int* hist,
-                              int hist_stride, const int* hist_len, int* out, hipStream_t stream) {
+                              int hist_stride, const int* hist_len, int small_k, int* out, hipStream_t stream) {
     ROCML_REQUIRE(batch >= 0 && vocab > 0, "sample: bad sizes B=%d V=%d", batch, vocab);
     ROCML_REQUIRE(logits && work && temperature && uniform && out, "sample: null argument");
     ROCML_REQUIRE(vocab <= SAMPLE_MAX_VOCAB, "sample: vocabulary %d exceeds %d", vocab, SAMPLE_MAX_VOCAB);
+    ROCML_REQUIRE(small_k >= 0 && small_k <= SMALL_K && (small_k == 0 || top_k), "sample: bad top-k bound %d", small_k);
     if (batch == 0) return 0;
+    if (small_k > 0) {
+        // slices of 4096 values (16 per thread), or of 16384 for the largest vocabularies
+        int ept = vocab <= MAX_SLICES * SLICE_THREADS * 16 ? 16 : 64;
+        int slice_len = SLICE_THREADS * ept;
+        int n_slices = (vocab + slice_len - 1) / slice_len;
+        if (n_slices <= MAX_SLICES && (long long)n_slices * small_k * 8 <= (long long)vocab * 4) {
+            float* cand_v = work;
+            int* cand_i = (int*)(work + (size_t)batch * n_slices * small_k);
+            dim3 grid(n_slices, batch);
+            if (ept == 16)
+                sample_slice_topk_kernel<16><<<grid, SLICE_THREADS, 0, stream>>>(
+                    logits, vocab, slice_len, temperature, top_k, penalty, hist, hist_stride, hist_len, small_k, cand_v, cand_i);
+            else
+                sample_slice_topk_kernel<64><<<grid, SLICE_THREADS, 0, stream>>>(
+                    logits, vocab, slice_len, temperature, top_k, penalty, hist, hist_stride, hist_len, small_k, cand_v, cand_i);
+            sample_merge_draw_kernel<<<batch, 64, 0, stream>>>(cand_v, cand_i, n_slices, small_k, temperature, top_k,
+                                                               top_p, uniform, out);
+            ROCML_CHECK_LAUNCH("sample");
+            return 0;
+        }
+    }
     sample_kernel<<<batch, SAMPLE_THREADS, 0, stream>>>(logits, work, vocab, temperature, top_k, top_p, uniform,
                                             penalty, hist, hist_stride, hist_len, out);
     ROCML_CHECK_LAUNCH("sample");

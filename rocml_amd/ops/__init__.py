@@ -44,7 +44,7 @@ _SIGNATURES = {
                             _P, _I, _I, _I, _I, _I, _P, _LL, _P],
     },
     "sampling": {
-        "rocml_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P],
+        "rocml_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _P],
         "rocml_argmax": [_P, _I, _I, _P, _P, _P],
     },
 }
@@ -327,6 +327,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache
 
 # ---- sampling ------------------------------------------------------------------------
 ARGMAX_WORK_WORDS = 64      # 32-bit words of workspace per row for the two-stage argmax
+SAMPLE_SMALL_K = 64         # the largest top-k that the slice kernels of the sampler take
 
 
 def argmax(logits: torch.Tensor, out: torch.Tensor, work: Optional[torch.Tensor] = None) -> None:
@@ -344,7 +345,10 @@ def argmax(logits: torch.Tensor, out: torch.Tensor, work: Optional[torch.Tensor]
 def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor,
            out: torch.Tensor, top_k: Optional[torch.Tensor] = None, top_p: Optional[torch.Tensor] = None,
            penalty: Optional[torch.Tensor] = None, history: Optional[torch.Tensor] = None,
-           history_len: Optional[torch.Tensor] = None) -> None:
+           history_len: Optional[torch.Tensor] = None, small_k: int = 0) -> None:
+    """``small_k``: 0, or a bound of at most 64 such that every sequence with a positive
+    temperature has its top_k in ``[1, small_k]``: the caller's promise, which lets the selection
+    run on slices of the vocabulary instead of whole rows."""
     _dev(logits, work, temperature, uniform, out, top_k, top_p, penalty, history, history_len)
     _want(logits, torch.float32, "logits")
     _want(work, torch.float32, "sampling workspace")
@@ -364,4 +368,4 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, 
     _check("sampling", library("sampling").rocml_sample(
         _ptr(logits), _ptr(work), batch, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform),
         _ptr(penalty), _ptr(history), 0 if history is None else history.shape[1], _ptr(history_len),
-        _ptr(out), _stream()))
+        int(small_k), _ptr(out), _stream()))

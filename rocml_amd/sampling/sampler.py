@@ -74,9 +74,12 @@ class DeviceSampler:
             top_k[b] = 0 if p.top_k is None else max(1, int(p.top_k))
             top_p[b] = -1.0 if p.top_p is None else min(max(float(p.top_p), 0.0), 1.0)
             uniform[b] = s.rng.next_f32()
+        # every drawing sequence with a small top-k: the selection may run on slices of the row
+        drawing = top_k[temperature > 0]
+        small_k = int(drawing.max()) if drawing.size and drawing.min() >= 1 and drawing.max() <= ops.SAMPLE_SMALL_K else 0
         floats = torch.from_numpy(np.stack([temperature, uniform, top_p, penalty])).to(self.device)
         ints = torch.from_numpy(np.concatenate([top_k, hist_len, hist.reshape(-1)])).to(self.device)
         ops.sample(logits, self._work, floats[0], floats[1], out, top_k=ints[:batch], top_p=floats[2],
                    penalty=floats[3], history=ints[2 * batch:].view(batch, window),
-                   history_len=ints[batch:2 * batch])
+                   history_len=ints[batch:2 * batch], small_k=small_k)
         return out.cpu().tolist()

@@ -109,6 +109,32 @@ def test_draws_follow_the_filtered_distribution(params):
         assert len(set(got)) == 1                          # the nucleus keeps at least one token
 
 
+@pytest.mark.parametrize("vocab", [700, 5000, 151936, 300001])
+@pytest.mark.parametrize("params", [
+    SamplingParams(temperature=0.9, top_k=1), SamplingParams(temperature=0.9, top_k=7, top_p=0.8),
+    SamplingParams(temperature=1.4, top_k=64, top_p=0.97, repeat_penalty=1.3),
+    SamplingParams(temperature=1.4, top_k=65, top_p=0.97, repeat_penalty=1.3)])
+def test_small_top_k_on_slices_of_the_row(vocab, params):
+    """A top-k of at most 64 is selected on slices of the vocabulary and merged by one wave, 65
+    by the kernel that walks whole rows: both against the plain rule, at vocabularies of one
+    slice, of a few, of many, and beyond the size where the slices grow."""
+    g = torch.Generator().manual_seed(vocab % 97)
+    batch = 32
+    logits = torch.randn(1, vocab, generator=g) * 2.0
+    logits[0, vocab - 1] = logits[0].max() + 0.5          # the last token of the last slice is a candidate
+    history = [int(t) for t in logits[0].topk(12).indices] * 2 + [int(t) for t in torch.randint(0, vocab, (30,), generator=g)]
+    p = candidates(logits[0].numpy(), params.temperature, params.top_k, params.top_p,
+                   params.repeat_penalty, history, params.repeat_penalty_window)
+    cum = np.cumsum(p)
+    us = [(i + 0.61) / batch for i in range(batch)]
+    got = _draw(logits.expand(batch, vocab).contiguous(), [params] * batch, us, [history] * batch)
+    for u, tok in zip(us, got):
+        assert p[tok] > 0, f"token {tok} is outside the candidate set"
+        t = u * cum[-1]
+        assert cum[tok] - p[tok] - 1e-4 * cum[-1] <= t <= cum[tok] + 1e-4 * cum[-1], (u, tok)
+    assert len(set(got)) <= params.top_k
+
+
 def test_ties_at_the_kth_value_keep_the_lowest_ids():
     logits = torch.full((1, 300), -5.0)
     logits[0, [10, 50, 90, 130]] = 2.0                      # four equal candidates, k = 2
