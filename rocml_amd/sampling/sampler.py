@@ -39,6 +39,20 @@ class DeviceSampler:
         self.device = torch.device(device)
         self._work: Optional[torch.Tensor] = None
         self._argmax_work: Optional[torch.Tensor] = None
+        # the parameters of a call travel in one pinned buffer and one copy (32-bit words, floats
+        # and integers side by side), the drawn ids come back through another
+        self._stage: Optional[torch.Tensor] = None
+        self._stage_dev: Optional[torch.Tensor] = None
+        self._ids_host: Optional[torch.Tensor] = None
+
+    def _ids(self, out: torch.Tensor) -> List[int]:
+        batch = out.numel()
+        if self._ids_host is None or self._ids_host.numel() < batch:
+            self._ids_host = torch.empty(max(batch, 64), dtype=torch.int32, pin_memory=True)
+        host = self._ids_host[:batch]
+        host.copy_(out, non_blocking=True)
+        torch.cuda.current_stream(self.device).synchronize()
+        return host.tolist()
 
     def sample(self, logits: torch.Tensor, seqs: Sequence[SequenceSampling]) -> List[int]:
         """``logits`` is ``[B, V]`` 32-bit on the device, row ``b`` for ``seqs[b]``.  Returns
@@ -50,17 +64,20 @@ class DeviceSampler:
             if self._argmax_work is None or self._argmax_work.numel() < batch * ops.ARGMAX_WORK_WORDS:
                 self._argmax_work = torch.empty(max(batch, 64) * ops.ARGMAX_WORK_WORDS, dtype=torch.int32, device=self.device)
             ops.argmax(logits, out, self._argmax_work)
-            return out.cpu().tolist()
+            return self._ids(out)
         if self._work is None or self._work.numel() < logits.numel():
             self._work = torch.empty(logits.numel(), dtype=torch.float32, device=self.device)
-        temperature = np.zeros(batch, np.float32)
-        uniform = np.zeros(batch, np.float32)
-        top_k = np.zeros(batch, np.int32)
-        top_p = np.full(batch, -1.0, np.float32)
-        penalty = np.zeros(batch, np.float32)
         window = max([s.params.repeat_penalty_window for s in seqs if s.params.penalty_active()] + [1])
-        hist = np.zeros((batch, window), np.int32)
-        hist_len = np.zeros(batch, np.int32)
+        words = batch * (6 + window)
+        if self._stage is None or self._stage.numel() < words:
+            self._stage = torch.empty(2 * words, dtype=torch.int32, pin_memory=True)
+            self._stage_dev = torch.empty(2 * words, dtype=torch.int32, device=self.device)
+        stage = self._stage[:words].numpy()
+        stage[:] = 0
+        temperature, uniform, top_p, penalty = (stage[i * batch:(i + 1) * batch].view(np.float32) for i in range(4))
+        top_k, hist_len = stage[4 * batch:5 * batch], stage[5 * batch:6 * batch]
+        hist = stage[6 * batch:].reshape(batch, window)
+        top_p[:] = -1.0
         for b, s in enumerate(seqs):
             p = s.params
             if p.penalty_active():
@@ -77,9 +94,11 @@ class DeviceSampler:
         # every drawing sequence with a small top-k: the selection may run on slices of the row
         drawing = top_k[temperature > 0]
         small_k = int(drawing.max()) if drawing.size and drawing.min() >= 1 and drawing.max() <= ops.SAMPLE_SMALL_K else 0
-        floats = torch.from_numpy(np.stack([temperature, uniform, top_p, penalty])).to(self.device)
-        ints = torch.from_numpy(np.concatenate([top_k, hist_len, hist.reshape(-1)])).to(self.device)
-        ops.sample(logits, self._work, floats[0], floats[1], out, top_k=ints[:batch], top_p=floats[2],
-                   penalty=floats[3], history=ints[2 * batch:].view(batch, window),
-                   history_len=ints[batch:2 * batch], small_k=small_k)
-        return out.cpu().tolist()
+        dev = self._stage_dev[:words]
+        dev.copy_(self._stage[:words], non_blocking=True)
+        floats = dev[:4 * batch].view(torch.float32)
+        ops.sample(logits, self._work, floats[:batch], floats[batch:2 * batch], out,
+                   top_k=dev[4 * batch:5 * batch], top_p=floats[2 * batch:3 * batch],
+                   penalty=floats[3 * batch:4 * batch], history=dev[6 * batch:].view(batch, window),
+                   history_len=dev[5 * batch:6 * batch], small_k=small_k)
+        return self._ids(out)
