@@ -98,28 +98,28 @@ template <int MT, int EPI>
 static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m, int n,
                          int k, void* workspace, long long workspace_bytes, SplitPlan plan, hipStream_t stream) {
     constexpr int LDS = 2 * MT * 16 * GS_ROW * 16;
-    // Waves per block.  The activations of a K chunk take LDS in proportion to the rows, and LDS
-    // decides how many blocks a CU holds: with 64 rows two.  Eight waves per block then double
-    // the weight bytes in flight per CU and halve the times the activations are read.  One row
-    // tile without a split (wide products) gets two waves: more, smaller blocks keep more loads
-    // in flight when nothing else multiplies their number.
-    constexpr int WIDE = MT == 4 ? 8 : 4;
-    constexpr bool CAN_NARROW = MT == 1;
-    constexpr bool DEEP = MT == 4;                    // weights two chunks ahead (gemm_skinny_deep_kernel)
+    // Up to 16 rows: four waves per block, or two for the wide products that cannot be split
+    // (more, smaller blocks keep more loads in flight when nothing else multiplies their
+    // number), about 512 blocks.  Beyond 16 rows the kernel that requests two steps ahead, with
+    // eight waves per block (LDS for the activations limits a CU to two blocks at 64 rows;
+    // eight waves double the weight bytes in flight per CU and halve the times the activations
+    // are read), about 256 blocks.
+    constexpr bool AHEAD = MT > 1;
+    constexpr int WIDE = AHEAD ? 8 : 4;
     static bool ready = false;
     if (!ready) {
-        if constexpr (DEEP) {
-            if (allow_lds(gemm_skinny_deep_kernel<MT, EPI, false, WIDE>, LDS, "gemm")) return 1;
-            if (allow_lds(gemm_skinny_deep_kernel<MT, EPI, true, WIDE>, LDS, "gemm")) return 1;
+        if constexpr (AHEAD) {
+            if (allow_lds(gemm_skinny_ahead_kernel<MT, EPI, false, WIDE>, LDS, "gemm")) return 1;
+            if (allow_lds(gemm_skinny_ahead_kernel<MT, EPI, true, WIDE>, LDS, "gemm")) return 1;
         } else {
             if (allow_lds(gemm_skinny_kernel<MT, EPI, false, WIDE>, LDS, "gemm")) return 1;
             if (allow_lds(gemm_skinny_kernel<MT, EPI, true, WIDE>, LDS, "gemm")) return 1;
         }
         ready = true;
     }
-    bool narrow = CAN_NARROW && (EPI == EPI_SWIGLU || n >= 65536);
+    bool narrow = !AHEAD && (EPI == EPI_SWIGLU || n >= 65536);
     int blocks_n = ceil_div(n, narrow ? 32 : 16 * WIDE);
-    int target = MT == 4 ? 256 : 512;
+    int target = AHEAD ? 256 : 512;
     int splits = target / blocks_n;
     int by_k = k / 512;
     if (splits > by_k) splits = by_k;
@@ -133,19 +133,19 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
     splits = ceil_div(k, k_per_split);
     dim3 grid(blocks_n, splits);
     if (splits == 1 && narrow) {
-        if constexpr (CAN_NARROW)
+        if constexpr (!AHEAD)
             gemm_skinny_kernel<MT, EPI, false, 2><<<grid, 128, LDS, stream>>>(
                 (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
     } else if (splits == 1) {
-        if constexpr (DEEP)
-            gemm_skinny_deep_kernel<MT, EPI, false, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
+        if constexpr (AHEAD)
+            gemm_skinny_ahead_kernel<MT, EPI, false, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
                 (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
         else
             gemm_skinny_kernel<MT, EPI, false, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
                 (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
     } else {
-        if constexpr (DEEP)
-            gemm_skinny_deep_kernel<MT, EPI, true, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
+        if constexpr (AHEAD)
+            gemm_skinny_ahead_kernel<MT, EPI, true, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
                 (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, workspace, n, m, n, k, k_per_split);
         else
             gemm_skinny_kernel<MT, EPI, true, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
@@ -202,6 +202,7 @@ static int launch_skinny_m(const void* x, int ldx, const void* w, int ldw, void*
                            int k, void* workspace, long long workspace_bytes, SplitPlan plan, hipStream_t stream) {
     if (m <= 16) return launch_skinny<1, EPI>(x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
     if (m <= 32) return launch_skinny<2, EPI>(x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
+    if (m <= 48) return launch_skinny<3, EPI>(x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
     return launch_skinny<4, EPI>(x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
 }
 

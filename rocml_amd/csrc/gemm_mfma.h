@@ -19,8 +19,8 @@
 //    workspace and are added in split order by a second kernel (or by the caller's next
 //    kernel), so results do not depend on timing
 //    (rocml-kernels/kernels/gemm_splitk_reduce.hip:4-10 has the same rule).
-//    gemm_skinny_deep_kernel is the same with weights requested two chunks ahead, for blocks
-//    of 64 rows.
+//    gemm_skinny_ahead_kernel is the same for 17 to 64 rows, with weights and activations
+//    requested two steps ahead.
 //  * gemm_kpar_kernel, one or two rows: the waves of a block split K and meet once in LDS.
 #pragma once
 #include "common.h"
@@ -372,111 +372,142 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restri
     skinny_epilogue<MT, EPI, PARTIAL>(acc, out, ldo, m, n, n0, lane, blockIdx.y);
 }
 
-// The same product for blocks of 64 rows, where the chip holds few waves (LDS for the
-// activations limits a CU to two blocks): weights are requested two chunks ahead instead of one,
-// so that a wave always has 8 to 16 loads of 16 bytes outstanding.  (For fewer rows, with four
-// times the blocks per CU, the deeper pipeline only lengthens the start and was slower.)
+// The same product for 17 to 64 rows.  With more rows a step costs more (four products and four
+// LDS reads per weight fragment at 64 rows) and the chip holds fewer waves, so what a step waits
+// for decides: here nothing in the loop waits for a load younger than a whole step.  The weights
+// of step c+2 are requested when the products of step c have been issued (into the registers
+// these have just read), the activations of step c+2 at the start of step c, and they are
+// written to the other LDS buffer at the end of step c+1.  (Everything requested before the
+// first product, four steps deep, was measured too: the waves then sit in the issue queue until
+// the data has all but arrived.)
+// All loads are buffer loads: the hardware returns zeros for an offset beyond the buffer, which
+// takes the place of every clamp and branch (rows beyond N or M, pieces beyond the K range,
+// whole steps beyond the last) and leaves the compiler's wait counts exact; a lane's address is
+// one 32-bit register for all of its loads.  A block's weight rows are its buffer, so only the
+// bytes of 16 * WAVES rows must fit 31 bits.
+constexpr uint32_t GA_NOWHERE = 0x80000000u;         // an offset beyond any buffer here
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t ga_buffer(const void* base, long long bytes) {
+    // raw buffer (stride 0), 32-bit data format; the range check is on the byte offset
+    return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)min(bytes, (long long)0x7fffffff), 0x00020000);
+}
+
 template <int MT, int EPI, bool PARTIAL, int WAVES>
 __global__ void __launch_bounds__(64 * WAVES)
-gemm_skinny_deep_kernel(const bf16_t* x, int ldx, const bf16_t* w, int ldw,
-                   void* out, int ldo, int m, int n, int k, int k_per_split) {
-    // (no __restrict__: a load from memory that is promised not to change may be moved anywhere,
-    // and the order of the loads below is the point)
+gemm_skinny_ahead_kernel(const bf16_t* x, int ldx, const bf16_t* w, int ldw, void* out, int ldo, int m, int n,
+                         int k, int k_per_split) {
     extern __shared__ u32x4_t gs_smem[];              // [2][MT*16][GS_ROW]
     constexpr int ROWS = MT * 16;
     constexpr int THREADS = 64 * WAVES;
-    constexpr int XCHUNKS = ROWS * (GS_KC / 8) / THREADS;   // 16-byte pieces per thread
+    constexpr int XL = ROWS * (GS_KC / 8) / THREADS;  // activation loads per thread and step
+    constexpr int D = 2;                              // steps that the weights are requested ahead
+    static_assert(XL >= 1 && ROWS * (GS_KC / 8) % THREADS == 0, "activation pieces must divide among the threads");
     int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    int n0 = blockIdx.x * (16 * WAVES) + wave * 16;
+    int block_row = blockIdx.x * (16 * WAVES);
+    int n0 = block_row + wave * 16;
     int ks = blockIdx.y * k_per_split;
     int ke = min(k, ks + k_per_split);
-    int n_chunks = (ke - ks + GS_KC - 1) / GS_KC;
-    const bf16_t* wsafe = w + (size_t)min(n0 + (lane & 15), n - 1) * ldw;
-    const bf16_t* wbase = wsafe + (lane >> 4) * 8;
-    u32x4_t w0[8], w1[8], w2[8], xr[XCHUNKS];
+    int n_steps = (ke - ks + GS_KC - 1) / GS_KC;
+    int rows_here = min(16 * WAVES, n - block_row);
+    __amdgpu_buffer_rsrc_t wbuf = ga_buffer(w + (size_t)block_row * ldw, ((long long)(rows_here - 1) * ldw + k) * 2);
+    __amdgpu_buffer_rsrc_t xbuf = ga_buffer(x, ((long long)(m - 1) * ldx + k) * 2);
+    // byte offsets of a lane's first piece: weight row lane%16 of the wave's tile, K piece lane/16
+    uint32_t woff = ((uint32_t)(wave * 16 + (lane & 15)) * (uint32_t)ldw + (lane >> 4) * 8) * 2;
+    uint32_t xoff[XL];
+    int xk[XL];                                       // K offset of activation piece i within a step
+#pragma unroll
+    for (int i = 0; i < XL; ++i) {
+        int piece = tid + i * THREADS;
+        xk[i] = (piece % (GS_KC / 8)) * 8;
+        xoff[i] = ((uint32_t)(piece / (GS_KC / 8)) * (uint32_t)ldx + xk[i]) * 2;
+    }
+    u32x4_t wr[D][8], xr[2][XL];
     f32x4_t acc[MT];
 #pragma unroll
     for (int i = 0; i < MT; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    // Blocks start their K loop at different chunks and wrap around: row strides are often a
+    // Blocks start their K loop at different steps and wrap around: row strides are often a
     // power of two, and blocks that all read the same K window at once would queue up on a few
     // memory channels.
-    int rot = (blockIdx.x * 5 + blockIdx.y * 3) % n_chunks;
-    // chunk c_ of the loop (clamped to the last one: loads past the end fetch something valid
-    // that nobody uses, so that no load stands under a branch)
-#define GD_CHUNK_BASE(c_) (ks + ((min((c_), n_chunks - 1) + rot) >= n_chunks ? min((c_), n_chunks - 1) + rot - n_chunks : min((c_), n_chunks - 1) + rot) * GS_KC)
-#define GD_LOAD_W(c_, dst_)                                                                     \
-    {                                                                                           \
-        int kb_ = GD_CHUNK_BASE(c_);                                                            \
-        _Pragma("unroll") for (int j = 0; j < 8; ++j) {                                         \
-            bool in_ = kb_ + j * 32 + (lane >> 4) * 8 < ke;                                     \
-            dst_[j] = *(const u32x4_t*)(in_ ? wbase + kb_ + j * 32 : wsafe);                    \
-        }                                                                                       \
-    }
-#define GD_LOAD_X(c_)                                                                           \
-    {                                                                                           \
-        int kb_ = GD_CHUNK_BASE(c_);                                                            \
-        _Pragma("unroll") for (int i = 0; i < XCHUNKS; ++i) {                                   \
-            int piece_ = tid + i * THREADS;                                                     \
-            int row_ = piece_ / (GS_KC / 8), gk_ = kb_ + (piece_ % (GS_KC / 8)) * 8;            \
-            xr[i] = *(const u32x4_t*)(gk_ < ke ? x + (size_t)min(row_, m - 1) * ldx + gk_ : x); \
-        }                                                                                       \
-    }
-#define GD_STORE_X(c_, buf_)                                                                    \
-    {                                                                                           \
-        int kb_ = GD_CHUNK_BASE(c_);                                                            \
-        u32x4_t* sx_ = gs_smem + (buf_) * ROWS * GS_ROW;                                        \
-        const u32x4_t zero_ = {0u, 0u, 0u, 0u};                                                 \
-        _Pragma("unroll") for (int i = 0; i < XCHUNKS; ++i) {                                   \
-            int piece_ = tid + i * THREADS;                                                     \
-            int kc_ = piece_ % (GS_KC / 8);                                                     \
-            sx_[(piece_ / (GS_KC / 8)) * GS_ROW + kc_] = kb_ + kc_ * 8 < ke ? xr[i] : zero_;    \
-        }                                                                                       \
-    }
-    // One chunk: the activations of the next chunk and the weights of the chunk after it are
-    // requested (in this order: loads return in order, and the activations are needed first),
-    // the products of this chunk run on weights that were requested two chunks ago, then the
-    // activations go to the other LDS buffer.  Weight loads stay in flight across the barrier:
-    // a wave always has 8 to 16 of them outstanding, which is what keeps the memory busy when
-    // the number of waves is small for the chip.
+    int rot = (blockIdx.x * 5 + blockIdx.y * 3) % n_steps;
+#define GA_BASE(c_) (ks + (((c_) + rot) >= n_steps ? (c_) + rot - n_steps : (c_) + rot) * GS_KC)
     // (neither the optimizer nor the scheduler may move a load across this)
-#define GD_KEEP_ORDER asm volatile("" ::: "memory"); __builtin_amdgcn_sched_barrier(0);
-#define GD_STEP(c_, wcur_, wfar_)                                                               \
+#define GA_KEEP_ORDER asm volatile("" ::: "memory"); __builtin_amdgcn_sched_barrier(0);
+    // (weights beyond the K range are not multiplied by zero but not loaded: a row's stride may
+    // be longer than K, and what lies between is anything)
+#define GA_LOAD_W(c_, set_)                                                                     \
     {                                                                                           \
-        GD_LOAD_X((c_) + 1)                                                                     \
-        GD_KEEP_ORDER                                                                           \
-        GD_LOAD_W((c_) + 2, wfar_)                                                              \
-        GD_KEEP_ORDER                                                                           \
-        const u32x4_t* sx = gs_smem + ((c_) & 1) * ROWS * GS_ROW;                               \
+        int kb_ = GA_BASE(c_);                                                                  \
+        bool step_ = (c_) < n_steps;                                                            \
         _Pragma("unroll") for (int j = 0; j < 8; ++j) {                                         \
-            bf16x8_t a = as_frag4(wcur_[j]);                                                    \
-            _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                 \
-                bf16x8_t b = as_frag4(sx[(mt * 16 + (lane & 15)) * GS_ROW + j * 4 + (lane >> 4)]); \
-                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);      \
-            }                                                                                   \
+            bool in_ = step_ && kb_ + j * 32 + (lane >> 4) * 8 < ke;                            \
+            wr[set_][j] = __builtin_amdgcn_raw_buffer_load_b128(                                \
+                wbuf, in_ ? woff + (uint32_t)kb_ * 2 + j * 64 : GA_NOWHERE, 0, 0);              \
         }                                                                                       \
-        GD_STORE_X((c_) + 1, ((c_) & 1) ^ 1)                                                    \
-        __syncthreads();                                                                        \
     }
-
-    GD_LOAD_W(0, w0)
-    GD_LOAD_X(0)
-    GD_STORE_X(0, 0)
-    GD_LOAD_W(1, w1)
+#define GA_LOAD_X(c_, set_)                                                                     \
+    {                                                                                           \
+        int kb_ = GA_BASE(c_);                                                                  \
+        bool step_ = (c_) < n_steps;                                                            \
+        _Pragma("unroll") for (int i = 0; i < XL; ++i) {                                        \
+            bool in_ = step_ && kb_ + xk[i] < ke;                                               \
+            xr[set_][i] = __builtin_amdgcn_raw_buffer_load_b128(                                \
+                xbuf, in_ ? xoff[i] + (uint32_t)kb_ * 2 : GA_NOWHERE, 0, 0);                    \
+        }                                                                                       \
+    }
+    // step c lives in register set and LDS buffer c % 2
+#define GA_STORE_X(set_)                                                                        \
+    {                                                                                           \
+        u32x4_t* sx_ = gs_smem + (set_) * ROWS * GS_ROW;                                        \
+        _Pragma("unroll") for (int i = 0; i < XL; ++i) {                                        \
+            int piece_ = tid + i * THREADS;                                                     \
+            sx_[(piece_ / (GS_KC / 8)) * GS_ROW + piece_ % (GS_KC / 8)] = xr[set_][i];          \
+        }                                                                                       \
+    }
+    GA_LOAD_X(0, 0)
+    GA_KEEP_ORDER
+    GA_LOAD_W(0, 0)
+    GA_KEEP_ORDER
+    GA_LOAD_X(1, 1)
+    GA_KEEP_ORDER
+    GA_LOAD_W(1, 1)
+    GA_KEEP_ORDER
+    GA_STORE_X(0)
     __syncthreads();
-    for (int c = 0; c < n_chunks; c += 3) {
-        GD_STEP(c, w0, w2)
-        if (c + 1 >= n_chunks) break;
-        GD_STEP(c + 1, w1, w0)
-        if (c + 2 >= n_chunks) break;
-        GD_STEP(c + 2, w2, w1)
+    for (int c0 = 0; c0 < n_steps; c0 += D) {
+#pragma unroll
+        for (int u = 0; u < D; ++u) {
+            int c = c0 + u;
+            if (c >= n_steps) break;
+            // the activations of step c+2 take the registers that step c's were stored from
+            GA_LOAD_X(c + 2, u)
+            GA_KEEP_ORDER
+            const u32x4_t* sx = gs_smem + u * ROWS * GS_ROW;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                bf16x8_t a = as_frag4(wr[u][j]);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    bf16x8_t b = as_frag4(sx[(mt * 16 + (lane & 15)) * GS_ROW + j * 4 + (lane >> 4)]);
+                    acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
+                }
+            }
+            // (a product has no side effect and would be sunk below the loads that follow, which
+            // then could not take the registers it reads: tie the sums to this place)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) asm volatile("" : "+v"(acc[mt]));
+            GA_KEEP_ORDER
+            GA_LOAD_W(c + D, u)
+            GA_KEEP_ORDER
+            GA_STORE_X(u ^ 1)
+            __syncthreads();
+        }
     }
-#undef GD_STEP
-#undef GD_KEEP_ORDER
-#undef GD_CHUNK_BASE
-#undef GD_LOAD_W
-#undef GD_LOAD_X
-#undef GD_STORE_X
+#undef GA_BASE
+#undef GA_KEEP_ORDER
+#undef GA_LOAD_W
+#undef GA_LOAD_X
+#undef GA_STORE_X
     skinny_epilogue<MT, EPI, PARTIAL>(acc, out, ldo, m, n, n0, lane, blockIdx.y);
 }
 

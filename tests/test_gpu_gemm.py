@@ -35,7 +35,7 @@ def test_plain_float32(m, n, k):
     assert float((acc.double() - (ref + base.double())).abs().max()) < 1e-5 * max(1.0, float(ref.abs().max()))
 
 
-SHAPES = [(1, 64, 64), (5, 200, 72), (16, 130, 512), (17, 96, 264), (33, 4096, 1024), (64, 257, 4096),
+SHAPES = [(1, 64, 64), (5, 200, 72), (16, 130, 512), (17, 96, 264), (33, 4096, 1024), (48, 1000, 776), (64, 257, 4096),
           (8, 1000, 2056), (128, 128, 64), (129, 300, 200), (300, 515, 72), (2048, 512, 1024)]
 
 
@@ -80,7 +80,7 @@ def test_strided_rows_and_refusals():
 
 
 @pytest.mark.parametrize("algo", [PLAIN, TILE, SKINNY, KPAR, TILE256])
-@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (7, 448, 96), (64, 1000, 264), (130, 256, 128), (300, 2048, 512)])
+@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (7, 448, 96), (25, 300, 520), (41, 130, 1032), (64, 1000, 264), (130, 256, 128), (300, 2048, 512)])
 def test_gated_epilogue(m, n, k, algo):
     """Rows of the weight are (gate, up) pairs; the output is silu(gate) * up, formed from
     the 32-bit sums."""
