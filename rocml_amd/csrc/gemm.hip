@@ -272,7 +272,11 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
     int epi = gated ? EPI_SWIGLU : accumulate ? EPI_ACC : (out_dtype == ROCML_BF16 ? EPI_BF16 : EPI_F32);
     bool use_mfma = mfma_ok && algo != ALGO_PLAIN;
     if (use_mfma) {
-        bool skinny = algo == ALGO_MFMA_SKINNY || (algo == ALGO_AUTO && m <= 64);
+        // Up to 16 rows the few-rows kernels; up to 64 rows still for the gated product (it cannot
+        // cut K in pieces, which is what the tile kernel lives on with so few rows) and, up to 32
+        // rows, for every product but the widest (the output projection over the vocabulary).
+        bool few_rows = m <= 16 || (m <= 64 && (gated || (m <= 32 && n < 65536)));
+        bool skinny = algo == ALGO_MFMA_SKINNY || (algo == ALGO_AUTO && few_rows);
         SplitPlan plan{defer, deferred_splits};
         int rc;
 #define BY_EPI(fn, ...)                                              \
