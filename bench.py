@@ -100,17 +100,15 @@ def main() -> int:
     def decode(batch: int, steps: int, warmup: int):
         slots = [engine.new_sequence() for _ in range(batch)]
         greedy = [SequenceSampling.start(SamplingParams.greedy(), i, []) for i in range(batch)]
-        # Prompts go in a few at a time: the prefill is not what is timed here.
+        # All prompts in one step, as the generation loop sends them (the engine cuts the step
+        # into pieces of its own; the prefill is not what is timed here).
         if args.skip_prompts:
             engine.cache.reserve(slots, [PROMPT_LEN] * batch)
             engine.cache.commit(slots, [PROMPT_LEN] * batch)
             tokens = [1] * batch
         else:
-            logits_rows = []
-            for i in range(0, batch, 4):
-                part = slots[i:i + 4]
-                logits_rows.append(engine.step([StepEntry(s, prompt(), [PROMPT_LEN - 1]) for s in part]).clone())
-            tokens = sampler.sample(torch.cat(logits_rows), greedy)
+            logits = engine.step([StepEntry(s, prompt(), [PROMPT_LEN - 1]) for s in slots])
+            tokens = sampler.sample(logits, greedy)
 
         def one_step(toks):
             logits = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, toks)])

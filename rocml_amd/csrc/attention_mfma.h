@@ -63,10 +63,10 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     const int* pages = block_table + (size_t)token_seq[t] * bt_width;
     int first_page = lo / AM_PAGE;
     int n_pages = (len + AM_PAGE - 1) / AM_PAGE - first_page;
-    int per_split = (n_pages + n_splits - 1) / n_splits;
-    int p_begin = first_page + split * per_split;
-    int p_end = min(first_page + n_pages, p_begin + per_split);
-    int n_pieces = max(0, p_end - p_begin) * 2;
+    // split s takes pages s, s + n_splits, ...: the splits of a sequence, which run side by side,
+    // then read neighbouring pages at any one time instead of n_splits distant ranges
+    int my_pages = split < n_pages ? (n_pages - split + n_splits - 1) / n_splits : 0;
+    int n_pieces = my_pages * 2;
 
     // Q^T operand: column = head of the group (zero beyond it), 8 values of D per lane and step.
     bf16x8_t qf[KD];
@@ -87,7 +87,7 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
 
     for (int piece = wave; piece < n_pieces; piece += 4) {
         // (the page index is the same for all lanes: a scalar load)
-        int lpage = __builtin_amdgcn_readfirstlane(p_begin + (piece >> 1)), half = piece & 1;
+        int lpage = __builtin_amdgcn_readfirstlane(first_page + split + (piece >> 1) * n_splits), half = piece & 1;
         int phys = pages[lpage];
         const bf16_t* kbase = kcache + (((size_t)phys * hkv + kvh) * AM_PAGE + half * 32) * D;
         const bf16_t* vbase = vcache + ((size_t)phys * hkv + kvh) * D * AM_PAGE + half * 32;
