@@ -283,7 +283,12 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
         (epi == EPI_F32 ? fn<EPI_F32>(__VA_ARGS__)                   \
          : epi == EPI_BF16 ? fn<EPI_BF16>(__VA_ARGS__)               \
          : epi == EPI_ACC ? fn<EPI_ACC>(__VA_ARGS__) : fn<EPI_SWIGLU>(__VA_ARGS__))
-        bool kpar = algo == ALGO_MFMA_KPAR || (algo == ALGO_AUTO && m <= 2);   // beyond two rows the activations read from L2 cost more than the block sharing of the few-rows kernel
+        // One or two rows: the kernel whose waves split K, unless the output is narrow (4096 or
+        // 5120 wide, the products that return to the hidden size): its blocks of 16 weight rows
+        // are then so few that K must be cut across blocks as well and a wave is left with one
+        // chunk; the few-rows kernel is 10 to 15 % faster there.  Beyond two rows the activations
+        // read from L2 cost more than the block sharing of the few-rows kernel.
+        bool kpar = algo == ALGO_MFMA_KPAR || (algo == ALGO_AUTO && m <= 2 && n >= 6144);
         if (kpar) rc = BY_EPI(launch_kpar, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
         else if (skinny) rc = BY_EPI(launch_skinny_m, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
         else rc = BY_EPI(launch_mfma_tile, x, ldx, w, ldw, out, ldo, m, n, k,
