@@ -67,6 +67,24 @@ def test_pages_follow_lengths_and_reserve_is_all_or_nothing():
     c.check()
 
 
+def test_sequences_of_a_step_get_neighbouring_pages():
+    """A step's sequences take their pages a page per sequence and round: page p of all of them
+    lies side by side in the pool, and a longer sequence goes on alone."""
+    c = _cache([FULL], 64 * 16)
+    s = [c.new_sequence() for _ in range(3)]
+    c.reserve(s, [130, 64, 200])               # 3, 1 and 4 pages
+    c.commit(s, [130, 64, 200])
+    g = c.kv_groups[0]
+    t = [g.page_table(x) for x in s]
+    assert [len(x) for x in t] == [3, 1, 4]
+    assert sorted([t[0][0], t[1][0], t[2][0]]) == [0, 1, 2]       # first pages of all three
+    assert sorted([t[0][1], t[2][1]]) == [3, 4] and sorted([t[0][2], t[2][2]]) == [5, 6]
+    assert t[2][3] == 7
+    c.reserve(s, [193, 65, 257])               # one more page each: again side by side
+    assert sorted([t[0][3], t[1][1], t[2][4]]) == [8, 9, 10]
+    c.check()
+
+
 def test_window_releases_pages_no_query_can_see():
     c = _cache([WIN], 64 * 8)
     s = c.new_sequence()
