@@ -117,7 +117,9 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
         }
         ready = true;
     }
-    bool narrow = !AHEAD && (EPI == EPI_SWIGLU || n >= 65536);
+    // (two waves per block also for the gated product of 17 to 32 rows: 9 % there)
+    constexpr bool CAN_NARROW = MT <= 2;
+    bool narrow = MT == 1 ? (EPI == EPI_SWIGLU || n >= 65536) : (MT == 2 && EPI == EPI_SWIGLU);
     int blocks_n = ceil_div(n, narrow ? 32 : 16 * WIDE);
     int target = AHEAD ? 256 : 512;
     int splits = target / blocks_n;
@@ -133,7 +135,10 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
     splits = ceil_div(k, k_per_split);
     dim3 grid(blocks_n, splits);
     if (splits == 1 && narrow) {
-        if constexpr (!AHEAD)
+        if constexpr (CAN_NARROW && AHEAD)
+            gemm_skinny_ahead_kernel<MT, EPI, false, 2><<<grid, 128, LDS, stream>>>(
+                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
+        else if constexpr (CAN_NARROW)
             gemm_skinny_kernel<MT, EPI, false, 2><<<grid, 128, LDS, stream>>>(
                 (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
     } else if (splits == 1) {
