@@ -142,7 +142,7 @@ rmsnorm_vec_kernel(float* x, const float* __restrict__ gain, TO* __restrict__ ou
             for (int q = 0; q < GROUP; ++q)
 #pragma unroll
                 for (int j = 0; j < RN_VEC; ++j) {
-                    if (threadIdx.x + j * EW_BLOCK >= nv || sp + q >= n_splits) continue;
+                    if ((int)threadIdx.x + j * EW_BLOCK >= nv || sp + q >= n_splits) continue;
                     v[j].x += a[q][j].x; v[j].y += a[q][j].y; v[j].z += a[q][j].z; v[j].w += a[q][j].w;
                 }
         }

@@ -291,6 +291,7 @@ sample_kernel(const float* __restrict__ logits, float* __restrict__ work, int vo
             __syncthreads();
             unsigned* mine = hist_cnt + (tid / 64) * 256;
             SAMPLE_ROW_PASS(wrow, vocab, work_vec, i, v,
+                (void)i;
                 uint32_t key = float_key(v);
                 if (level == 0 || (key >> (shift + 8)) == found) atomicAdd(mine + ((key >> shift) & 255), 1u);
             )
