@@ -27,17 +27,28 @@ struct AttnArgs {
     const int* cu_seqlens; int n_seqs; int n_tokens; int total_q_tiles; int max_len;
     int hq, hkv; float scale; int window; void* workspace; long long workspace_bytes;
     int n_splits_hint;
+    const DecodeProj* proj;     // decode only: the step's q/k/v projection instead of q and an appended cache
 };
 
-template <int D>
-static int launch_decode(const AttnArgs& a, hipStream_t stream) {
+template <int D, bool FUSED, int AHEAD>
+static int launch_decode_kernel(const AttnArgs& a, int n_splits, float* part_o, float* part_ml, hipStream_t stream) {
     int group = a.hq / a.hkv;
     int lds = 4 * group * (D + 4) * (int)sizeof(float);
     static int allowed = 0;
     if (lds > allowed) {
-        if (allow_lds(attn_decode_mfma_kernel<D>, lds)) return 1;
+        if (allow_lds(attn_decode_mfma_kernel<D, FUSED, AHEAD>, lds)) return 1;
         allowed = lds;
     }
+    dim3 grid(n_splits, a.hkv, a.n_tokens);
+    attn_decode_mfma_kernel<D, FUSED, AHEAD><<<grid, AM_THREADS, lds, stream>>>(
+        a.q, a.out, const_cast<bf16_t*>(a.kcache), const_cast<bf16_t*>(a.vcache), a.block_table, a.bt_width,
+        a.token_seq, a.token_pos, a.hq, a.hkv, a.scale * LOG2E, a.window, n_splits, part_o, part_ml,
+        FUSED ? *a.proj : DecodeProj{});
+    return 0;
+}
+
+template <int D, bool FUSED>
+static int launch_decode(const AttnArgs& a, hipStream_t stream) {
     // Enough blocks to fill the chip, at most one split per page of the longest sequence.
     int n_splits = a.n_splits_hint;
     if (n_splits <= 0) {
@@ -53,15 +64,23 @@ static int launch_decode(const AttnArgs& a, hipStream_t stream) {
     if (n_splits < 1) n_splits = 1;
     float* part_o = (float*)a.workspace;
     float* part_ml = part_o ? part_o + (size_t)a.n_tokens * a.hq * n_splits * D : nullptr;
-    dim3 grid(n_splits, a.hkv, a.n_tokens);
-    attn_decode_mfma_kernel<D><<<grid, AM_THREADS, lds, stream>>>(
-        a.q, a.out, a.kcache, a.vcache, a.block_table, a.bt_width, a.token_seq, a.token_pos, a.hq, a.hkv,
-        a.scale * LOG2E, a.window, n_splits, part_o, part_ml);
+    // Many splits mean few pieces per block: then two of a wave's pieces travel at a time.  The
+    // choice follows the launch's shape, not the lengths, as the number of splits does.
+    int rc;
+    if constexpr (D <= 128)
+        rc = n_splits >= 4 ? launch_decode_kernel<D, FUSED, 2>(a, n_splits, part_o, part_ml, stream)
+                           : launch_decode_kernel<D, FUSED, 1>(a, n_splits, part_o, part_ml, stream);
+    else
+        rc = launch_decode_kernel<D, FUSED, 1>(a, n_splits, part_o, part_ml, stream);
+    if (rc) return rc;
     if (n_splits > 1)
         // whole waves: the kernel's reductions exchange values between all 64 lanes
         attn_decode_reduce_kernel<D><<<a.n_tokens * a.hq, (D + 63) / 64 * 64, 0, stream>>>(part_o, part_ml, a.out, n_splits);
     return 0;
 }
+
+template <int D> static int launch_decode_plain(const AttnArgs& a, hipStream_t s) { return launch_decode<D, false>(a, s); }
+template <int D> static int launch_decode_fused(const AttnArgs& a, hipStream_t s) { return launch_decode<D, true>(a, s); }
 
 template <int D>
 static int launch_prefill(const AttnArgs& a, hipStream_t stream) {
@@ -117,8 +136,8 @@ ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, c
     if (mfma_ok && algo != ATTN_PLAIN) {
         AttnArgs a{(const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table,
                    bt_width, token_seq, token_pos, cu_seqlens, n_seqs, n_tokens, total_q_tiles, max_len, hq, hkv,
-                   scale, window, workspace, workspace_bytes, n_splits};
-        int rc = decode ? BY_HEAD_DIM(launch_decode, d, a, stream) : BY_HEAD_DIM(launch_prefill, d, a, stream);
+                   scale, window, workspace, workspace_bytes, n_splits, nullptr};
+        int rc = decode ? BY_HEAD_DIM(launch_decode_plain, d, a, stream) : BY_HEAD_DIM(launch_prefill, d, a, stream);
         if (rc) return rc;
         ROCML_CHECK_LAUNCH("attention");
         return 0;
@@ -136,5 +155,50 @@ ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, c
     else
         return rocml_fail("attention: unknown dtype code %d", dtype);
     ROCML_CHECK_LAUNCH("attention");
+    return 0;
+}
+
+// A decode step's attention straight from the q/k/v projection: per-head norm, rotation, append
+// to the cache and attention in one launch (and the merge of the splits in a second), instead of
+// a kernel for the first three and rocml_attention for the rest.  One token per sequence;
+// bfloat16 cache with pages of 64 positions; a head size of 64, 128, 192 or 256; at most 16
+// query heads per kv head.  qkv is the projection's 32-bit output [tokens, ld] with q, k and v
+// side by side (k and v are not read when write_kv is 0: the cache then holds this step's row
+// already), or its split-K partial sums [qkv_splits][tokens][ld], which are added in split
+// order.  q_gain/k_gain null: no norm; cos/sin null: no rotation, else [tokens, D/2].
+ROCML_EXPORT int rocml_attention_decode_fused(const float* qkv, int ld, int qkv_splits, long long qkv_split_stride,
+                                              const float* q_gain, const float* k_gain, float eps,
+                                              const float* cos_t, const float* sin_t, int write_kv, void* out,
+                                              void* kcache, void* vcache, const int* block_table, int bt_width,
+                                              const int* token_seq, const int* token_pos, int n_tokens, int hq,
+                                              int hkv, int d, int page_size, float scale, int window,
+                                              int max_len, int n_splits, void* workspace,
+                                              long long workspace_bytes, hipStream_t stream) {
+    ROCML_REQUIRE(n_tokens >= 0 && hq > 0 && hkv > 0 && bt_width > 0 && qkv_splits >= 1,
+                  "fused decode attention: bad sizes T=%d Hq=%d Hkv=%d width=%d splits=%d", n_tokens, hq, hkv,
+                  bt_width, qkv_splits);
+    ROCML_REQUIRE(hq % hkv == 0 && hq / hkv <= 16,
+                  "fused decode attention: %d query heads over %d kv heads (at most 16 per kv head)", hq, hkv);
+    ROCML_REQUIRE(page_size == AM_PAGE && (d == 64 || d == 128 || d == 192 || d == 256),
+                  "fused decode attention: needs pages of 64 positions and a head size of 64, 128, 192 or 256 "
+                  "(page=%d D=%d)", page_size, d);
+    ROCML_REQUIRE(window >= 0, "fused decode attention: negative window %d", window);
+    int rows = write_kv ? hq + 2 * hkv : hq;
+    ROCML_REQUIRE(ld >= rows * d && ld % 4 == 0 && ((uintptr_t)qkv & 15) == 0 &&
+                      (qkv_splits == 1 || (qkv_split_stride >= (long long)n_tokens * ld && qkv_split_stride % 4 == 0)),
+                  "fused decode attention: projection rows of %d values (need %d, a multiple of 4, 16-byte aligned), "
+                  "split stride %lld", ld, rows * d, qkv_split_stride);
+    ROCML_REQUIRE((q_gain == nullptr) == (k_gain == nullptr) && (cos_t == nullptr) == (sin_t == nullptr),
+                  "fused decode attention: gains and rotation tables come in pairs");
+    if (n_tokens == 0) return 0;
+    DecodeProj pj{qkv, ld, qkv_splits, qkv_split_stride, q_gain, k_gain, eps, cos_t, sin_t, write_kv};
+    AttnArgs a{nullptr, (bf16_t*)out, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table, bt_width,
+               token_seq, token_pos, nullptr, 0, n_tokens, 0, max_len, hq, hkv, scale, window, workspace,
+               workspace_bytes, n_splits, &pj};
+    int rc = d == 64 ? launch_decode_fused<64>(a, stream)
+             : d == 128 ? launch_decode_fused<128>(a, stream)
+             : d == 192 ? launch_decode_fused<192>(a, stream) : launch_decode_fused<256>(a, stream);
+    if (rc) return rc;
+    ROCML_CHECK_LAUNCH("fused decode attention");
     return 0;
 }

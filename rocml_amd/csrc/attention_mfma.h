@@ -40,16 +40,49 @@ __device__ __forceinline__ float sum_across_halves(float v) {
 }
 
 // ---- decode: one query token per sequence ----------------------------------------------------
+// What the fused decode kernel reads in place of finished q rows and an appended cache row: the
+// output of the q/k/v projection in 32-bit (or its split-K partial sums, [splits][tokens][ld]),
+// the gains of the per-head norm (null: no norm) and the rotation tables (null: no rotation;
+// else the whole head is rotated, pairs (e, e + D/2)).
+struct DecodeProj {
+    const float* qkv; int ld; int n_splits; long long split_stride;
+    const float* q_gain; const float* k_gain; float eps;
+    const float* cos_t; const float* sin_t; int write_kv;
+};
+
+// p[0] + p[stride] + ... in split order, four loads in flight at a time.
+__device__ __forceinline__ float sum_of_splits(const float* p, int n_splits, long long stride) {
+    float val = 0.f;
+    for (int sp = 0; sp < n_splits; sp += 4) {
+        float a0 = p[sp * stride];
+        float a1 = p[sp + 1 < n_splits ? (sp + 1) * stride : 0];
+        float a2 = p[sp + 2 < n_splits ? (sp + 2) * stride : 0];
+        float a3 = p[sp + 3 < n_splits ? (sp + 3) * stride : 0];
+        val += a0;
+        if (sp + 1 < n_splits) val += a1;
+        if (sp + 2 < n_splits) val += a2;
+        if (sp + 3 < n_splits) val += a3;
+    }
+    return val;
+}
+
 // grid (n_splits, Hkv, tokens), 4 waves; the block's pages are cut into 32-key pieces that the
 // waves take in turn; all query heads of the kv head ride in the 16 columns of the MFMA.
-template <int D>
+//
+// FUSED: the kernel takes the projection's output instead of q and a finished cache: every block
+// norms and rotates the q heads of its kv head itself, in the layout of the MFMA operand; the
+// block that owns the sequence's last page also norms and rotates the new key, writes it and the
+// new value into the cache and puts both into the registers of the piece that holds the new
+// position, where the loads from the cache may or may not have seen them yet.  A page belongs
+// to one split, so no other block reads that row in this launch.
+template <int D, bool FUSED, int AHEAD>
 __global__ void __launch_bounds__(AM_THREADS)
 attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
-                        const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
+                        bf16_t* kcache, bf16_t* vcache,
                         const int* __restrict__ block_table, int bt_width,
                         const int* __restrict__ token_seq, const int* __restrict__ token_pos, int hq,
                         int hkv, float scale_log2e, int window, int n_splits,
-                        float* __restrict__ part_o, float* __restrict__ part_ml) {
+                        float* __restrict__ part_o, float* __restrict__ part_ml, DecodeProj pj) {
     constexpr int KD = D / 32;      // MFMA steps along D for the scores
     constexpr int DT = D / 16;      // 16-row tiles of the output
     extern __shared__ float sm_o[];                 // [4 waves][group][D + 4]
@@ -68,39 +101,21 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     int my_pages = split < n_pages ? (n_pages - split + n_splits - 1) / n_splits : 0;
     int n_pieces = my_pages * 2;
 
-    // Q^T operand: column = head of the group (zero beyond it), 8 values of D per lane and step.
-    bf16x8_t qf[KD];
-    {
-        bool ok = col < group;
-        const bf16_t* qrow = q + ((size_t)t * hq + kvh * group + (ok ? col : 0)) * D + g * 8;
-#pragma unroll
-        for (int kd = 0; kd < KD; ++kd) {
-            uint4 v = *(const uint4*)(qrow + kd * 32);
-            v.x = ok ? v.x : 0u; v.y = ok ? v.y : 0u; v.z = ok ? v.z : 0u; v.w = ok ? v.w : 0u;
-            qf[kd] = __builtin_bit_cast(bf16x8_t, v);
-        }
-    }
-    float m = -INFINITY, l = 0.f;
-    f32x4_t o[DT];
-#pragma unroll
-    for (int i = 0; i < DT; ++i) o[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-
-    for (int piece = wave; piece < n_pieces; piece += 4) {
+    const bf16_t* knew_lds = nullptr;
+    const bf16_t* vnew_lds = nullptr;
+    // Row r of score tile u is key 8 (r / 4) + 4u + r % 4 of a piece: then the 8 keys whose
+    // probabilities a lane holds after the softmax (rows 4g .. 4g+3 of both tiles) are the
+    // consecutive keys 8g .. 8g+7, and its values for them are one 16-byte load.
+    // AHEAD = 2: two pieces are on their way at a time.  A block of a small batch has a piece or
+    // two per wave, and their trips to memory then overlap; long loops gain nothing from it and
+    // lose a block per CU to the registers.
+    uint4 kbuf[AHEAD][2][KD], vbuf[AHEAD][DT];
+    auto request_piece = [&](int piece, uint4 (&kreg)[2][KD], uint4 (&vreg)[DT]) {
         // (the page index is the same for all lanes: a scalar load)
         int lpage = __builtin_amdgcn_readfirstlane(first_page + split + (piece >> 1) * n_splits), half = piece & 1;
         int phys = pages[lpage];
         const bf16_t* kbase = kcache + (((size_t)phys * hkv + kvh) * AM_PAGE + half * 32) * D;
         const bf16_t* vbase = vcache + ((size_t)phys * hkv + kvh) * D * AM_PAGE + half * 32;
-        int key0 = lpage * AM_PAGE + half * 32;
-        // All loads of the piece go out before anything is computed, the values too: a block has
-        // few pieces, and keys, softmax, values one after the other would be two trips to memory
-        // per piece where one will do.  (Requesting the next piece while this one is multiplied
-        // was tried: with eight waves per CU the memory is busy anyway, and short sequences paid
-        // for the extra request at their end.)
-        // Row r of score tile u is key 8 (r / 4) + 4u + r % 4 of the piece: then the 8 keys whose
-        // probabilities a lane holds after the softmax (rows 4g .. 4g+3 of both tiles) are the
-        // consecutive keys 8g .. 8g+7, and its values for them are one 16-byte load.
-        uint4 kreg[2][KD], vreg[DT];
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const bf16_t* krow = kbase + (size_t)(8 * (col >> 2) + 4 * u + (col & 3)) * D + g * 8;
@@ -110,6 +125,127 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
             vreg[dt] = *(const uint4*)(vbase + (size_t)(dt * 16 + col) * AM_PAGE + g * 8);
+    };
+    // The wave's first pieces are requested before the queries: their keys and values travel
+    // together with them.
+    if (wave < n_pieces) request_piece(wave, kbuf[0], vbuf[0]);
+    if (AHEAD == 2 && wave + 4 < n_pieces) request_piece(wave + 4, kbuf[AHEAD - 1], vbuf[AHEAD - 1]);
+    // Q^T operand: column = head of the group (zero beyond it), 8 values of D per lane and step.
+    bf16x8_t qf[KD];
+    bool owner = false;      // this block appends the new key and value
+    int new_pos = len - 1;
+    if constexpr (!FUSED) {
+        bool ok = col < group;
+        const bf16_t* qrow = q + ((size_t)t * hq + kvh * group + (ok ? col : 0)) * D + g * 8;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) {
+            uint4 v = *(const uint4*)(qrow + kd * 32);
+            v.x = ok ? v.x : 0u; v.y = ok ? v.y : 0u; v.z = ok ? v.z : 0u; v.w = ok ? v.w : 0u;
+            qf[kd] = __builtin_bit_cast(bf16x8_t, v);
+        }
+    } else {
+        // Rows of the projection this block turns into operands: the q heads of its kv head and,
+        // in the block whose split holds the sequence's last page, the new key and value.  A wave
+        // takes a row at a time, a lane the values lane, lane + 64, ...; two rows per wave are
+        // loaded together, so a group of four heads with key and value is one trip to memory.
+        constexpr int J = D / 64;
+        __shared__ float sm_f[AM_THREADS / 64][2][D];                        // a row before its rotation
+        __shared__ __attribute__((aligned(16))) bf16_t sm_q[16 * D];        // [head of the group][D]
+        __shared__ __attribute__((aligned(16))) bf16_t sm_knew[D];
+        __shared__ __attribute__((aligned(16))) bf16_t sm_vnew[D];
+        int last_lpage = new_pos / AM_PAGE;
+        owner = pj.write_kv && (last_lpage - first_page) % n_splits == split;
+        int n_rows = group + (owner ? 2 : 0);       // q heads, then key, then value
+        const float* tok = pj.qkv + (size_t)t * pj.ld;
+        for (int base = 0; base < n_rows; base += 2 * (AM_THREADS / 64)) {
+            int r[2];
+            const float* src[2];
+            float raw[2][J][4];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                r[i] = base + i * (AM_THREADS / 64) + wave;
+                int prow = r[i] < group ? kvh * group + r[i] : (r[i] == group ? hq + kvh : hq + hkv + kvh);
+                src[i] = tok + (size_t)(r[i] < n_rows ? prow : 0) * D + lane;
+#pragma unroll
+                for (int j = 0; j < J; ++j)
+#pragma unroll
+                    for (int sp = 0; sp < 4; ++sp)
+                        raw[i][j][sp] = src[i][j * 64 + (sp < pj.n_splits ? sp * pj.split_stride : 0)];
+            }
+            float val[2][J];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                // split-K partial sums of the projection, added in split order
+#pragma unroll
+                for (int j = 0; j < J; ++j) {
+                    float a = raw[i][j][0];
+#pragma unroll
+                    for (int sp = 1; sp < 4; ++sp)
+                        if (sp < pj.n_splits) a += raw[i][j][sp];
+                    for (int sp = 4; sp < pj.n_splits; ++sp) a += src[i][j * 64 + sp * pj.split_stride];
+                    val[i][j] = a;
+                }
+                const float* gain = r[i] < group ? pj.q_gain : (r[i] == group ? pj.k_gain : nullptr);
+                if (gain) {
+                    float ss = 0.f;
+#pragma unroll
+                    for (int j = 0; j < J; ++j) ss = fmaf(val[i][j], val[i][j], ss);
+                    float inv = 1.0f / sqrtf(wave_sum(ss) / (float)D + pj.eps);
+#pragma unroll
+                    for (int j = 0; j < J; ++j) val[i][j] = val[i][j] * inv * gain[lane + j * 64];
+                }
+#pragma unroll
+                for (int j = 0; j < J; ++j) sm_f[wave][i][lane + j * 64] = val[i][j];
+            }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                if (r[i] >= n_rows) continue;
+                bool rotate = pj.cos_t != nullptr && r[i] <= group;
+                const float* c = pj.cos_t + (size_t)t * (D / 2);
+                const float* sn = pj.sin_t + (size_t)t * (D / 2);
+                bf16_t* dst = r[i] < group ? sm_q + r[i] * D : (r[i] == group ? sm_knew : sm_vnew);
+                int phys = pages[last_lpage], in_page = new_pos % AM_PAGE;
+#pragma unroll
+                for (int j = 0; j < J; ++j) {
+                    int e = lane + j * 64;
+                    float x = val[i][j];
+                    if (rotate) {
+                        if (e < D / 2) x = x * c[e] - sm_f[wave][i][e + D / 2] * sn[e];
+                        else x = sm_f[wave][i][e - D / 2] * sn[e - D / 2] + x * c[e - D / 2];
+                    }
+                    bf16_t xb = f32_to_bf16(x);
+                    dst[e] = xb;
+                    if (r[i] == group && phys >= 0)
+                        kcache[(((size_t)phys * hkv + kvh) * AM_PAGE + in_page) * D + e] = xb;
+                    if (r[i] == group + 1 && phys >= 0)
+                        vcache[(((size_t)phys * hkv + kvh) * D + e) * AM_PAGE + in_page] = xb;
+                }
+            }
+            __syncthreads();
+        }
+        {
+            bool ok = col < group;
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) {
+                uint4 v = *(const uint4*)(sm_q + (ok ? col : 0) * D + kd * 32 + g * 8);
+                v.x = ok ? v.x : 0u; v.y = ok ? v.y : 0u; v.z = ok ? v.z : 0u; v.w = ok ? v.w : 0u;
+                qf[kd] = __builtin_bit_cast(bf16x8_t, v);
+            }
+        }
+        knew_lds = sm_knew;
+        vnew_lds = sm_vnew;
+    }
+    float m = -INFINITY, l = 0.f;
+    f32x4_t o[DT];
+#pragma unroll
+    for (int i = 0; i < DT; ++i) o[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    // All loads of a piece go out before anything is computed, the values too: a block has
+    // few pieces, and keys, softmax, values one after the other would be two trips to memory
+    // per piece where one will do.
+    // keys [key0, key0 + 32) of which those in [from, to) count
+    auto multiply_piece = [&](int key0, int from, int to, const uint4 (&kreg)[2][KD], const uint4 (&vreg)[DT]) {
         __builtin_amdgcn_sched_barrier(0);
         // scores of 2 x 16 keys: element i of s[u] is key 8g + 4u + i, column = head.
         f32x4_t s[2];
@@ -126,7 +262,7 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 int key = key0 + g * 8 + u * 4 + i;
-                float v = (key >= lo && key < len) ? s[u][i] * scale_log2e : -INFINITY;
+                float v = (key >= from && key < to) ? s[u][i] * scale_log2e : -INFINITY;
                 s[u][i] = v;
                 mx = fmaxf(mx, v);
             }
@@ -155,6 +291,36 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         for (int dt = 0; dt < DT; ++dt) {
             o[dt] = o[dt] * corr;
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vreg[dt]), pf, o[dt], 0, 0, 0);
+        }
+    };
+    // (FUSED: the new key is not yet in the cache where a block reads it; it comes last, from LDS)
+    int cached = (FUSED && owner) ? new_pos : len;
+    auto first_key = [&](int piece) { return (first_page + split + (piece >> 1) * n_splits) * AM_PAGE + (piece & 1) * 32; };
+    for (int piece = wave; piece < n_pieces; piece += 4 * AHEAD) {
+        multiply_piece(first_key(piece), lo, cached, kbuf[0], vbuf[0]);
+        if (piece + 4 * AHEAD < n_pieces) request_piece(piece + 4 * AHEAD, kbuf[0], vbuf[0]);
+        if (AHEAD == 2 && piece + 4 < n_pieces) {
+            multiply_piece(first_key(piece + 4), lo, cached, kbuf[AHEAD - 1], vbuf[AHEAD - 1]);
+            if (piece + 12 < n_pieces) request_piece(piece + 12, kbuf[AHEAD - 1], vbuf[AHEAD - 1]);
+        }
+    }
+    if constexpr (FUSED) {
+        // The step's own key and value as a piece of their own, row 0 of score tile 0, in the
+        // wave whose turn would be next.
+        if (owner && wave == (n_pieces & 3)) {
+            bool krow = col == 0, vrow = g == 0;
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int kd = 0; kd < KD; ++kd) {
+                    uint4 v = *(const uint4*)(knew_lds + kd * 32 + g * 8);
+                    bool take = krow && u == 0;
+                    kbuf[0][u][kd] = make_uint4(take ? v.x : 0u, take ? v.y : 0u, take ? v.z : 0u, take ? v.w : 0u);
+                }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                vbuf[0][dt] = make_uint4(vrow ? (uint32_t)vnew_lds[dt * 16 + col] : 0u, 0u, 0u, 0u);
+            multiply_piece(new_pos, new_pos, new_pos + 1, kbuf[0], vbuf[0]);
         }
     }
     // merge the four waves in wave order; element i of o[dt] is d = 16 dt + 4g + i, column = head.

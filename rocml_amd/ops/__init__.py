@@ -42,6 +42,8 @@ _SIGNATURES = {
     "attention": {
         "rocml_attention": [_P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I,
                             _P, _I, _I, _I, _I, _I, _P, _LL, _P],
+        "rocml_attention_decode_fused": [_P, _I, _I, _LL, _P, _P, _F, _P, _P, _I, _P, _P, _P, _P, _I, _P, _P,
+                                         _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _LL, _P],
     },
     "sampling": {
         "rocml_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _P],
@@ -323,6 +325,68 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache
         block_table.shape[1], _ptr(token_seq), _ptr(token_pos), n_tokens, n_heads, n_kv_heads, head_dim,
         page, scale, 0 if window is None else int(window), algo, _ptr(cu_seqlens), n_seqs, max_new,
         total_q_tiles, max_len, n_splits, ws_ptr, ws_bytes, _stream()))
+
+
+FUSED_DECODE_HEAD_DIMS = (64, 128, 192, 256)
+
+
+def attention_decode_fusable(dtype: torch.dtype, n_heads: int, n_kv_heads: int, head_dim: int, page: int,
+                             rot_dim: Optional[int]) -> bool:
+    """Whether ``attention_decode_fused`` takes this layer: bfloat16 cache in pages of 64, a head
+    size it has a kernel for, at most 16 query heads per kv head, and a rotation (if any) of the
+    whole head."""
+    return (dtype == torch.bfloat16 and page == 64 and head_dim in FUSED_DECODE_HEAD_DIMS
+            and n_heads // n_kv_heads <= 16 and rot_dim in (None, head_dim))
+
+
+def attention_decode_fused(qkv: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                           block_table: torch.Tensor, token_seq: torch.Tensor, token_pos: torch.Tensor,
+                           n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
+                           q_gain: Optional[torch.Tensor], k_gain: Optional[torch.Tensor], eps: float,
+                           cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], write_kv: bool = True,
+                           window: Optional[int] = None, workspace: Optional[torch.Tensor] = None,
+                           max_len: int = 0, n_splits: int = 0) -> None:
+    """A decode step's attention straight from the q/k/v projection ``qkv`` (float32
+    ``[tokens, ld]``, or its split-K partial sums ``[splits, tokens, ld]``): per-head norm,
+    rotation, append of the new key and value to the cache and attention over the cache in one
+    launch.  ``workspace`` must not overlap ``qkv``."""
+    _dev(qkv, out, k_cache, v_cache, block_table, token_seq, token_pos, q_gain, k_gain, cos, sin)
+    _want(qkv, torch.float32, "projection output")
+    qkv_splits, split_stride = 1, 0
+    if qkv.dim() == 3:
+        qkv_splits, split_stride = qkv.shape[0], qkv.shape[1] * qkv.shape[2]
+        qkv = qkv[0]
+    n_tokens, ld = qkv.shape
+    page = k_cache.shape[2]
+    if not attention_decode_fusable(k_cache.dtype, n_heads, n_kv_heads, head_dim, page,
+                                    None if cos is None else 2 * cos.shape[-1]):
+        raise KernelError(f"fused decode attention does not take this layer (cache {k_cache.dtype}, pages of {page}, "
+                          f"head size {head_dim}, {n_heads} heads over {n_kv_heads})")
+    if out.shape != (n_tokens, n_heads * head_dim) or out.dtype != k_cache.dtype:
+        raise KernelError("attention output must be [tokens, heads * head_dim] of the cache's type")
+    if v_cache.dtype != k_cache.dtype or k_cache.shape[1:] != (n_kv_heads, page, head_dim) \
+            or v_cache.shape != (k_cache.shape[0], n_kv_heads, head_dim, page):
+        raise KernelError(f"cache {tuple(k_cache.shape)} / {tuple(v_cache.shape)} does not fit {n_kv_heads} heads of {head_dim}")
+    for g in (q_gain, k_gain):
+        if g is not None:
+            _want(g, torch.float32, "head norm gain")
+            if g.numel() != head_dim:
+                raise KernelError(f"head norm gain has {g.numel()} values for head size {head_dim}")
+    if cos is not None:
+        _want(cos, torch.float32, "rotation table")
+        if cos.shape != (n_tokens, head_dim // 2) or sin is None or sin.shape != cos.shape or sin.dtype != cos.dtype:
+            raise KernelError(f"rotation tables must be float32 {(n_tokens, head_dim // 2)}")
+    _want(block_table, torch.int32, "block table")
+    _want(token_seq, torch.int32, "token sequence table")
+    _want(token_pos, torch.int32, "token position table")
+    if token_seq.numel() != n_tokens or token_pos.numel() != n_tokens:
+        raise KernelError("one sequence index and one position per token are needed")
+    ws_ptr, ws_bytes = (None, 0) if workspace is None else (workspace.data_ptr(), workspace.numel() * workspace.element_size())
+    _check("attention", library("attention").rocml_attention_decode_fused(
+        _ptr(qkv), ld, qkv_splits, split_stride, _ptr(q_gain), _ptr(k_gain), eps, _ptr(cos), _ptr(sin),
+        1 if write_kv else 0, _ptr(out), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
+        _ptr(token_seq), _ptr(token_pos), n_tokens, n_heads, n_kv_heads, head_dim, page, scale,
+        0 if window is None else int(window), max_len, n_splits, ws_ptr, ws_bytes, _stream()))
 
 
 # ---- sampling ------------------------------------------------------------------------

@@ -87,16 +87,26 @@ class Attention(Mixer):
         if self.position is not None:
             cos, sin = self.position.tables(step)
             rot = self.position.rot_dim
-        q = ws.get("attn.q", (n, self.q_dim), self.dtype)
         eps = s.qk_norm.eps if s.qk_norm is not None else 1.0
-        ops.qk_norm_rope_append(qkv, s.n_heads, s.n_kv_heads, s.head_dim, self.q_gain, self.k_gain, eps,
-                                cos, sin, rot, q, cache.k, cache.v, cache.block_table, step.token_seq,
-                                step.token_pos, write_kv=owns_cache, n_splits=max(splits, 1))
         o = ws.get("attn.o", (n, self.q_dim), self.dtype)
-        ops.attention(q, o, cache.k, cache.v, cache.block_table, step.token_seq, step.token_pos,
-                      s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, workspace=ws.scratch(),
-                      cu_seqlens=step.cu_seqlens, max_new=step.max_new, total_q_tiles=step.total_q_tiles,
-                      max_len=step.max_len, n_splits=self._decode_splits(step, cache))
+        if step.max_new == 1 and ops.attention_decode_fusable(cache.k.dtype, s.n_heads, s.n_kv_heads, s.head_dim,
+                                                               cache.k.shape[2], rot if cos is not None else None):
+            # One token per sequence: norm, rotation, append and attention in one launch, straight
+            # from the projection.  The attention's own partial results go behind the projection's.
+            used = (splits * n * rows * 4 + 255) // 256 * 256 if splits else 0
+            ops.attention_decode_fused(qkv, o, cache.k, cache.v, cache.block_table, step.token_seq, step.token_pos,
+                                       s.n_heads, s.n_kv_heads, s.head_dim, s.scale, self.q_gain, self.k_gain, eps,
+                                       cos, sin, write_kv=owns_cache, window=s.window, workspace=scratch[used:],
+                                       max_len=step.max_len, n_splits=self._decode_splits(step, cache))
+        else:
+            q = ws.get("attn.q", (n, self.q_dim), self.dtype)
+            ops.qk_norm_rope_append(qkv, s.n_heads, s.n_kv_heads, s.head_dim, self.q_gain, self.k_gain, eps,
+                                    cos, sin, rot, q, cache.k, cache.v, cache.block_table, step.token_seq,
+                                    step.token_pos, write_kv=owns_cache, n_splits=max(splits, 1))
+            ops.attention(q, o, cache.k, cache.v, cache.block_table, step.token_seq, step.token_pos,
+                          s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, workspace=ws.scratch(),
+                          cu_seqlens=step.cu_seqlens, max_new=step.max_new, total_q_tiles=step.total_q_tiles,
+                          max_len=step.max_len, n_splits=self._decode_splits(step, cache))
         splits = ops.gemm(o, self.w_o, x_accum, accumulate=True, workspace=ws.scratch(), defer=True)
         if splits:
             ws.set_pending(x_accum, splits)

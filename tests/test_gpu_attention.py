@@ -163,6 +163,99 @@ def test_a_far_key_decides():
             assert float((got[:, h] - want[h // (hq // hkv)]).abs().max()) < 2e-2
 
 
+def _fused_case(seqs, hq, hkv, d, qkv_splits, attn_splits, window, seed, norm=True, rotate=True):
+    """A decode step through the fused kernel: random projection output (cut into partial sums),
+    gains and rotation angles; the position of every sequence's new token holds a large value in
+    the cache beforehand, so a row that is not replaced shows.  Checked against the two-kernel
+    path (same cache rows, same output within rounding of q) and against plain attention over
+    the keys and values computed here."""
+    dev, ks, vs, _ = _build(seqs, hq, hkv, d, torch.bfloat16, seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    n = len(seqs)
+    rows = (hq + 2 * hkv) * d
+    parts = torch.randn(qkv_splits, n, rows, generator=g) * (1.0 / math.sqrt(qkv_splits))
+    qkv = parts.double().sum(0)
+    q_gain = (1 + 0.3 * torch.randn(d, generator=g)) if norm else None
+    k_gain = (1 + 0.3 * torch.randn(d, generator=g)) if norm else None
+    eps = 1e-5
+    angle = torch.rand(n, d // 2, generator=g).double() * 6.28
+    cos, sin = (torch.cos(angle).float(), torch.sin(angle).float()) if rotate else (None, None)
+
+    def prepare(x, gain):          # [n, heads, d] in float64
+        if gain is not None:
+            x = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * gain.double()
+        if rotate:
+            c, s_ = cos.double()[:, None], sin.double()[:, None]
+            lo_, hi_ = x[..., :d // 2], x[..., d // 2:]
+            x = torch.cat([lo_ * c - hi_ * s_, lo_ * s_ + hi_ * c], dim=-1)
+        return x
+    q = prepare(qkv[:, :hq * d].reshape(n, hq, d), q_gain)
+    k_new = prepare(qkv[:, hq * d:(hq + hkv) * d].reshape(n, hkv, d), k_gain)
+    v_new = qkv[:, (hq + hkv) * d:].reshape(n, hkv, d)
+    scale = 1.0 / math.sqrt(d)
+    table = dev["table"].cpu()
+    for b, (length, _) in enumerate(seqs):      # spoil the new token's row
+        page, at = int(table[b, (length - 1) // PAGE]), (length - 1) % PAGE
+        dev["kc"][page, :, at] = 1e4
+        dev["vc"][page, :, :, at] = 1e4
+    cuda = lambda t: None if t is None else t.cuda()
+    ws = torch.empty(32 << 20, dtype=torch.uint8, device="cuda")
+    parts_dev = parts.cuda() if qkv_splits > 1 else parts[0].cuda()
+    max_len = max(length for length, _ in seqs)
+    # the two-kernel path on a copy of the cache
+    kc2, vc2 = dev["kc"].clone(), dev["vc"].clone()
+    q_dev = torch.empty(n, hq * d, dtype=torch.bfloat16, device="cuda")
+    out2 = torch.full_like(q_dev, float("nan"))
+    ops.qk_norm_rope_append(parts_dev, hq, hkv, d, cuda(q_gain), cuda(k_gain), eps, cuda(cos), cuda(sin),
+                            d if rotate else 0, q_dev, kc2, vc2, dev["table"], dev["tok_seq"], dev["tok_pos"],
+                            n_splits=qkv_splits)
+    ops.attention(q_dev, out2, kc2, vc2, dev["table"], dev["tok_seq"], dev["tok_pos"], hq, hkv, d, scale, window,
+                  algo=MFMA, workspace=ws, cu_seqlens=dev["cu"], max_new=1, total_q_tiles=n, max_len=max_len,
+                  n_splits=attn_splits)
+    out = torch.full_like(q_dev, float("nan"))
+    ops.attention_decode_fused(parts_dev, out, dev["kc"], dev["vc"], dev["table"], dev["tok_seq"], dev["tok_pos"],
+                               hq, hkv, d, scale, cuda(q_gain), cuda(k_gain), eps, cuda(cos), cuda(sin),
+                               window=window, workspace=ws, max_len=max_len, n_splits=attn_splits)
+    torch.cuda.synchronize()
+    # the cache: a 32-bit sum in another order may round a value to the neighbouring bfloat16
+    for got, want in ((dev["kc"], kc2), (dev["vc"], vc2)):
+        diff = (got.float() - want.float()).abs()
+        assert float((diff / want.float().abs().clamp_min(1e-3)).max()) < 1e-2
+    got = out.cpu().double().reshape(n, hq, d)
+    assert float((got - out2.cpu().double().reshape(n, hq, d)).abs().max()) < 2e-2
+    for b, ((length, _), k, v) in enumerate(zip(seqs, ks, vs)):
+        k = k.double().clone()
+        v = v.double().clone()
+        k[length - 1], v[length - 1] = k_new[b].bfloat16().double(), v_new[b].bfloat16().double()
+        ref = _reference(q[b:b + 1].bfloat16(), k, v, [length - 1], scale, window)
+        err = float((got[b:b + 1] - ref).abs().max())
+        assert err < 1.5e-2, f"sequence {b} of length {length}: error {err}"
+
+
+# (Hq, Hkv, D, context lengths, splits of the projection, splits of the keys, window)
+FUSED = [(16, 8, 128, [1], 1, 0, None), (16, 8, 128, [2, 33, 64, 65, 257], 1, 0, None),
+         (32, 8, 128, [2048, 700, 1, 129], 4, 8, None), (8, 2, 256, [400, 1024, 63], 2, 6, None),
+         (4, 1, 64, [130, 31, 32, 96, 97], 3, 2, None), (16, 1, 64, [65, 128], 1, 0, None),
+         (24, 3, 192, [500, 9], 5, 5, None), (8, 2, 128, [1, 64, 65, 700, 129, 2, 1000], 4, 5, 70),
+         (8, 2, 128, [1, 64, 65, 700, 129], 1, 3, 1), (6, 2, 64, [300, 5], 2, 0, 128)]
+
+
+@pytest.mark.parametrize("hq,hkv,d,lengths,qkv_splits,attn_splits,window", FUSED)
+def test_decode_fused_with_norm_rotation_and_append(hq, hkv, d, lengths, qkv_splits, attn_splits, window):
+    _fused_case([(n, 1) for n in lengths], hq, hkv, d, qkv_splits, attn_splits, window, seed=11)
+
+
+def test_decode_fused_without_norm_or_rotation():
+    _fused_case([(77, 1), (200, 1)], 8, 4, 128, 2, 3, None, seed=12, norm=False)
+    _fused_case([(77, 1), (200, 1)], 8, 4, 128, 1, 0, None, seed=13, rotate=False)
+
+
+def test_decode_fused_refuses_other_head_sizes():
+    from rocml_amd.errors import KernelError
+    with pytest.raises(KernelError):
+        _fused_case([(10, 1)], 4, 2, 96, 1, 0, None, seed=0)
+
+
 def test_refusals():
     from rocml_amd.errors import KernelError
     dev, *_ = _build([(10, 1)], 4, 2, 48, torch.bfloat16, 0)
