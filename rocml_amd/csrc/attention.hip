@@ -166,6 +166,7 @@ ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, c
 // side by side (k and v are not read when write_kv is 0: the cache then holds this step's row
 // already), or its split-K partial sums [qkv_splits][tokens][ld], which are added in split
 // order.  q_gain/k_gain null: no norm; cos/sin null: no rotation, else [tokens, D/2].
+// token_seq null: token t is the one token of the step's sequence t (row t of the block table).
 ROCML_EXPORT int rocml_attention_decode_fused(const float* qkv, int ld, int qkv_splits, long long qkv_split_stride,
                                               const float* q_gain, const float* k_gain, float eps,
                                               const float* cos_t, const float* sin_t, int write_kv, void* out,

@@ -91,9 +91,15 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     int g = lane >> 4, col = lane & 15;
     int group = hq / hkv;
+    // (token_seq null: token t is the one token of the step's sequence t)
+    const int* pages = block_table + (size_t)(token_seq ? token_seq[t] : t) * bt_width;
+    // Without a window a split's pages are split, split + n_splits, ... whatever the length: the
+    // first four are looked up together with the position, a trip to memory earlier.
+    int early[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) early[i] = pages[split + i * n_splits < bt_width ? split + i * n_splits : 0];
     int len = token_pos[t] + 1;
     int lo = window > 0 ? max(0, len - window) : 0;
-    const int* pages = block_table + (size_t)token_seq[t] * bt_width;
     int first_page = lo / AM_PAGE;
     int n_pages = (len + AM_PAGE - 1) / AM_PAGE - first_page;
     // split s takes pages s, s + n_splits, ...: the splits of a sequence, which run side by side,
@@ -112,8 +118,12 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     uint4 kbuf[AHEAD][2][KD], vbuf[AHEAD][DT];
     auto request_piece = [&](int piece, uint4 (&kreg)[2][KD], uint4 (&vreg)[DT]) {
         // (the page index is the same for all lanes: a scalar load)
-        int lpage = __builtin_amdgcn_readfirstlane(first_page + split + (piece >> 1) * n_splits), half = piece & 1;
-        int phys = pages[lpage];
+        int round = __builtin_amdgcn_readfirstlane(piece >> 1), half = piece & 1;
+        int phys;
+        if (window == 0 && round < 4)
+            phys = round == 0 ? early[0] : round == 1 ? early[1] : round == 2 ? early[2] : early[3];
+        else
+            phys = pages[first_page + split + round * n_splits];
         const bf16_t* kbase = kcache + (((size_t)phys * hkv + kvh) * AM_PAGE + half * 32) * D;
         const bf16_t* vbase = vcache + ((size_t)phys * hkv + kvh) * D * AM_PAGE + half * 32;
 #pragma unroll

@@ -340,7 +340,7 @@ def attention_decode_fusable(dtype: torch.dtype, n_heads: int, n_kv_heads: int, 
 
 
 def attention_decode_fused(qkv: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
-                           block_table: torch.Tensor, token_seq: torch.Tensor, token_pos: torch.Tensor,
+                           block_table: torch.Tensor, token_seq: Optional[torch.Tensor], token_pos: torch.Tensor,
                            n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
                            q_gain: Optional[torch.Tensor], k_gain: Optional[torch.Tensor], eps: float,
                            cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], write_kv: bool = True,
@@ -349,7 +349,8 @@ def attention_decode_fused(qkv: torch.Tensor, out: torch.Tensor, k_cache: torch.
     """A decode step's attention straight from the q/k/v projection ``qkv`` (float32
     ``[tokens, ld]``, or its split-K partial sums ``[splits, tokens, ld]``): per-head norm,
     rotation, append of the new key and value to the cache and attention over the cache in one
-    launch.  ``workspace`` must not overlap ``qkv``."""
+    launch.  ``token_seq`` None: token ``t`` is the one token of the step's sequence ``t`` (row
+    ``t`` of the block table).  ``workspace`` must not overlap ``qkv``."""
     _dev(qkv, out, k_cache, v_cache, block_table, token_seq, token_pos, q_gain, k_gain, cos, sin)
     _want(qkv, torch.float32, "projection output")
     qkv_splits, split_stride = 1, 0
@@ -377,9 +378,12 @@ def attention_decode_fused(qkv: torch.Tensor, out: torch.Tensor, k_cache: torch.
         if cos.shape != (n_tokens, head_dim // 2) or sin is None or sin.shape != cos.shape or sin.dtype != cos.dtype:
             raise KernelError(f"rotation tables must be float32 {(n_tokens, head_dim // 2)}")
     _want(block_table, torch.int32, "block table")
-    _want(token_seq, torch.int32, "token sequence table")
     _want(token_pos, torch.int32, "token position table")
-    if token_seq.numel() != n_tokens or token_pos.numel() != n_tokens:
+    if token_seq is not None:
+        _want(token_seq, torch.int32, "token sequence table")
+    elif block_table.shape[0] < n_tokens:
+        raise KernelError(f"the block table has {block_table.shape[0]} rows for {n_tokens} sequences")
+    if (token_seq is not None and token_seq.numel() != n_tokens) or token_pos.numel() != n_tokens:
         raise KernelError("one sequence index and one position per token are needed")
     ws_ptr, ws_bytes = (None, 0) if workspace is None else (workspace.data_ptr(), workspace.numel() * workspace.element_size())
     _check("attention", library("attention").rocml_attention_decode_fused(

@@ -94,7 +94,8 @@ class Attention(Mixer):
             # One token per sequence: norm, rotation, append and attention in one launch, straight
             # from the projection.  The attention's own partial results go behind the projection's.
             used = (splits * n * rows * 4 + 255) // 256 * 256 if splits else 0
-            ops.attention_decode_fused(qkv, o, cache.k, cache.v, cache.block_table, step.token_seq, step.token_pos,
+            # (a step of one token per sequence numbers its tokens as its sequences)
+            ops.attention_decode_fused(qkv, o, cache.k, cache.v, cache.block_table, None, step.token_pos,
                                        s.n_heads, s.n_kv_heads, s.head_dim, s.scale, self.q_gain, self.k_gain, eps,
                                        cos, sin, write_kv=owns_cache, window=s.window, workspace=scratch[used:],
                                        max_len=step.max_len, n_splits=self._decode_splits(step, cache))

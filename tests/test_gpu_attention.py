@@ -213,10 +213,17 @@ def _fused_case(seqs, hq, hkv, d, qkv_splits, attn_splits, window, seed, norm=Tr
                   algo=MFMA, workspace=ws, cu_seqlens=dev["cu"], max_new=1, total_q_tiles=n, max_len=max_len,
                   n_splits=attn_splits)
     out = torch.full_like(q_dev, float("nan"))
+    kc3, vc3 = dev["kc"].clone(), dev["vc"].clone()
     ops.attention_decode_fused(parts_dev, out, dev["kc"], dev["vc"], dev["table"], dev["tok_seq"], dev["tok_pos"],
                                hq, hkv, d, scale, cuda(q_gain), cuda(k_gain), eps, cuda(cos), cuda(sin),
                                window=window, workspace=ws, max_len=max_len, n_splits=attn_splits)
+    # without the sequence table: token t is sequence t, as in this step
+    out3 = torch.full_like(q_dev, float("nan"))
+    ops.attention_decode_fused(parts_dev, out3, kc3, vc3, dev["table"], None, dev["tok_pos"],
+                               hq, hkv, d, scale, cuda(q_gain), cuda(k_gain), eps, cuda(cos), cuda(sin),
+                               window=window, workspace=ws, max_len=max_len, n_splits=attn_splits)
     torch.cuda.synchronize()
+    assert torch.equal(out, out3) and torch.equal(kc3, dev["kc"]) and torch.equal(vc3, dev["vc"])
     # the cache: a 32-bit sum in another order may round a value to the neighbouring bfloat16
     for got, want in ((dev["kc"], kc2), (dev["vc"], vc2)):
         diff = (got.float() - want.float()).abs()
