@@ -375,34 +375,39 @@ template <int D>
 __global__ void attn_decode_reduce_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                           bf16_t* __restrict__ out, int n_splits) {
     // At most 64 splits: lane s of every wave fetches split s's maximum and sum, so the loads
-    // go out together; the weights then sit in LDS for the sum over splits.
+    // go out together; the weights then sit in LDS for the sum over splits.  The partial
+    // outputs of the first eight splits are requested before the weights are formed: the
+    // kernel is one trip to memory for them.  The block has at least D threads.
     __shared__ float wgt[64];
     int row = blockIdx.x;     // token * Hq + head
     const float* ml = part_ml + (size_t)row * n_splits * 2;
+    const float* po = part_o + (size_t)row * n_splits * D;
     int lane = threadIdx.x & 63;
+    int d = threadIdx.x < D ? threadIdx.x : 0;
     bool has = lane < n_splits;
     float ms = has ? ml[lane * 2] : -INFINITY;
     float ls = has ? ml[lane * 2 + 1] : 0.f;
+    float first[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) first[s] = po[(size_t)min(s, n_splits - 1) * D + d];
     float mm = wave_max(ms);
     float w = ms == -INFINITY ? 0.f : fast_exp2(ms - mm);
     if (threadIdx.x < 64) wgt[lane] = w;
     float inv_l = 1.0f / wave_sum(ls * w);          // every wave computes the same sum
     __syncthreads();
-    const float* po = part_o + (size_t)row * n_splits * D;
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
-        float acc = 0.f;
-        int s = 0;
-        for (; s + 4 <= n_splits; s += 4) {
-            float a0 = po[(size_t)s * D + d], a1 = po[(size_t)(s + 1) * D + d];
-            float a2 = po[(size_t)(s + 2) * D + d], a3 = po[(size_t)(s + 3) * D + d];
-            acc += a0 * wgt[s];
-            acc += a1 * wgt[s + 1];
-            acc += a2 * wgt[s + 2];
-            acc += a3 * wgt[s + 3];
-        }
-        for (; s < n_splits; ++s) acc += po[(size_t)s * D + d] * wgt[s];
-        out[(size_t)row * D + d] = f32_to_bf16(acc * inv_l);
+    // (splits beyond the last have weight zero, and their loads are aimed at the last split's
+    // finite values: no branches)
+    float acc = 0.f;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) acc += first[s] * wgt[s];
+    for (int s0 = 8; s0 < n_splits; s0 += 8) {
+        float more[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) more[s] = po[(size_t)min(s0 + s, n_splits - 1) * D + d];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) acc += more[s] * wgt[s0 + s];
     }
+    if (threadIdx.x < D) out[(size_t)row * D + d] = f32_to_bf16(acc * inv_l);
 }
 
 // ---- prefill: many query tokens per sequence --------------------------------------------------
