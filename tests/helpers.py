@@ -58,8 +58,16 @@ TINY_G = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "vocab_s
           "rope_theta": 10000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": False,
           "max_position_embeddings": 512, "hidden_act": "silu", "attention_bias": False}
 
+# A head size of 128 on three key/value heads of two query heads each, no window: in bfloat16 the
+# decode steps of this one (and of D) take the attention kernel that reads the projection itself.
+TINY_H = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "vocab_size": 777,
+          "hidden_size": 88, "intermediate_size": 120, "num_hidden_layers": 2,
+          "num_attention_heads": 6, "num_key_value_heads": 3, "head_dim": 128,
+          "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": False,
+          "max_position_embeddings": 1024, "hidden_act": "silu", "attention_bias": False}
+
 TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3), "E": (TINY_E, 4), "F": (TINY_F, 5),
-        "G": (TINY_G, 22)}
+        "G": (TINY_G, 22), "H": (TINY_H, 23)}
 
 
 def make_model_dir(tmp_path, config: Dict, seed: int, dtype=torch.float32) -> str:

@@ -11,7 +11,7 @@ from tests import helpers
 
 
 def test_reads_every_size_from_config_json():
-    for cfg in (helpers.TINY_A, helpers.TINY_B, helpers.TINY_C, helpers.TINY_D, helpers.TINY_E, helpers.TINY_F, helpers.TINY_G):
+    for cfg in (helpers.TINY_A, helpers.TINY_B, helpers.TINY_C, helpers.TINY_D, helpers.TINY_E, helpers.TINY_F, helpers.TINY_G, helpers.TINY_H):
         c = Qwen3Config.from_dict(cfg)
         for key in ("vocab_size", "hidden_size", "intermediate_size", "num_hidden_layers",
                     "num_attention_heads", "num_key_value_heads", "head_dim", "rope_theta", "rms_norm_eps",

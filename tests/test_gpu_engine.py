@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 # Largest absolute difference over the largest absolute logit.
 TOL = {"float32": 2e-5, "bfloat16": 2e-2}
 LENGTHS = {"A": [5, 9, 13, 100], "B": [1, 7, 16, 33, 130], "C": [3, 24, 25, 70, 97], "D": [2, 64, 65, 150],
-           "E": [1, 40, 129], "F": [70, 150], "G": [12, 95, 76]}
+           "E": [1, 40, 129], "F": [70, 150], "G": [12, 95, 76], "H": [7, 65, 200, 321]}
 
 
 @pytest.fixture(scope="module")
@@ -40,7 +40,7 @@ def _oracle_weights(weights, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F", "G"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F", "G", "H"])
 def test_whole_tail_and_batches(models, name, dtype):
     path, cfg, weights = models[name]
     engine = _engine(path, dtype)
