@@ -257,6 +257,38 @@ def test_decode_fused_without_norm_or_rotation():
     _fused_case([(77, 1), (200, 1)], 8, 4, 128, 1, 0, None, seed=13, rotate=False)
 
 
+def test_decode_fused_one_key_decides():
+    """The projection is made so that one key carries almost all weight: first the step's own
+    key, which never comes from the cache, then a key far back in it.  The output must be that
+    key's value row."""
+    hq, hkv, d, length = 8, 2, 128, 900
+    for own in (True, False):
+        for splits in (0, 1, 7):
+            dev, ks, vs, _ = _build([(length, 1)], hq, hkv, d, torch.bfloat16, 7)
+            far = 37
+            qkv = torch.zeros(1, (hq + 2 * hkv) * d)
+            qkv[0, :hq * d].view(hq, d)[:, 5] = 40.0
+            v_new = torch.randn(hkv, d, generator=torch.Generator().manual_seed(3))
+            qkv[0, (hq + hkv) * d:] = v_new.reshape(-1)
+            if own:
+                qkv[0, hq * d:(hq + hkv) * d].view(hkv, d)[:, 5] = 40.0
+                want = v_new.bfloat16().double()
+            else:
+                page = int(dev["table"][0, far // PAGE])
+                k_row = torch.zeros(hkv, d)
+                k_row[:, 5] = 40.0
+                dev["kc"][page, :, far % PAGE] = k_row.to(torch.bfloat16).cuda()
+                want = vs[0][far].double()
+            out = torch.full((1, hq * d), float("nan"), dtype=torch.bfloat16, device="cuda")
+            ws = torch.empty(8 << 20, dtype=torch.uint8, device="cuda")
+            ops.attention_decode_fused(qkv.cuda(), out, dev["kc"], dev["vc"], dev["table"], None, dev["tok_pos"],
+                                       hq, hkv, d, 1.0, None, None, 1.0, None, None, workspace=ws,
+                                       max_len=length, n_splits=splits)
+            got = out.cpu().double().reshape(hq, d)
+            for h in range(hq):
+                assert float((got[h] - want[h // (hq // hkv)]).abs().max()) < 2e-2, (own, splits, h)
+
+
 def test_decode_fused_refuses_other_head_sizes():
     from rocml_amd.errors import KernelError
     with pytest.raises(KernelError):
