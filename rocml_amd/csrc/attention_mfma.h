@@ -50,31 +50,15 @@ struct DecodeProj {
     const float* cos_t; const float* sin_t; int write_kv;
 };
 
-// p[0] + p[stride] + ... in split order, four loads in flight at a time.
-__device__ __forceinline__ float sum_of_splits(const float* p, int n_splits, long long stride) {
-    float val = 0.f;
-    for (int sp = 0; sp < n_splits; sp += 4) {
-        float a0 = p[sp * stride];
-        float a1 = p[sp + 1 < n_splits ? (sp + 1) * stride : 0];
-        float a2 = p[sp + 2 < n_splits ? (sp + 2) * stride : 0];
-        float a3 = p[sp + 3 < n_splits ? (sp + 3) * stride : 0];
-        val += a0;
-        if (sp + 1 < n_splits) val += a1;
-        if (sp + 2 < n_splits) val += a2;
-        if (sp + 3 < n_splits) val += a3;
-    }
-    return val;
-}
-
 // grid (n_splits, Hkv, tokens), 4 waves; the block's pages are cut into 32-key pieces that the
 // waves take in turn; all query heads of the kv head ride in the 16 columns of the MFMA.
 //
 // FUSED: the kernel takes the projection's output instead of q and a finished cache: every block
-// norms and rotates the q heads of its kv head itself, in the layout of the MFMA operand; the
-// block that owns the sequence's last page also norms and rotates the new key, writes it and the
-// new value into the cache and puts both into the registers of the piece that holds the new
-// position, where the loads from the cache may or may not have seen them yet.  A page belongs
-// to one split, so no other block reads that row in this launch.
+// norms and rotates the q heads of its kv head itself and lays them out as the MFMA operand; the
+// block whose split holds the sequence's last page also norms and rotates the new key, writes it
+// and the new value into the cache and multiplies them as one more piece, from LDS: the loads
+// from the cache may or may not see a row that is written in the same launch, so the cached
+// keys end before it.  A page belongs to one split, so no other block reads that row.
 template <int D, bool FUSED, int AHEAD>
 __global__ void __launch_bounds__(AM_THREADS)
 attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
