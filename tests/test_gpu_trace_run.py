@@ -35,9 +35,9 @@ def logits_of(out_dir, step, vocab):
     return torch.from_numpy(np.fromfile(os.path.join(out_dir, f"{step}.f32"), dtype="<f4").reshape(-1, vocab))
 
 
-@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 2e-2)])
-def test_replay_whole_tail_and_batches(tmp_path, dtype, tol):
-    cfg, seed = helpers.TINY["B"]
+@pytest.mark.parametrize("name,dtype,tol", [("B", "float32", 2e-5), ("B", "bfloat16", 2e-2), ("H", "bfloat16", 2e-2)])
+def test_replay_whole_tail_and_batches(tmp_path, name, dtype, tol):
+    cfg, seed = helpers.TINY[name]
     path = helpers.make_model_dir(tmp_path, cfg, seed, torch.float32)
     weights = helpers.read_weights(path)
     if dtype == "bfloat16":
