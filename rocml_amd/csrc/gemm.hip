@@ -9,7 +9,7 @@
 ROCML_LAST_ERROR_FN(gemm)
 
 enum GemmAlgo : int { ALGO_AUTO = 0, ALGO_PLAIN = 1, ALGO_MFMA_TILE = 2, ALGO_MFMA_SKINNY = 3, ALGO_MFMA_KPAR = 4,
-                      ALGO_MFMA_TILE256 = 5 };
+                      ALGO_MFMA_TILE256 = 5, ALGO_MFMA_TILE192 = 6 };
 
 static int round_up(int a, int b) { return (a + b - 1) / b * b; }
 
@@ -55,11 +55,13 @@ static int launch_mfma_tile_as(const void* x, int ldx, const void* w, int ldw, v
     return 0;
 }
 
-// shape: 0 = choose, 1 = 128x128 tiles, 2 = 256x256.  The choice is made on an estimate of the
-// time.  A CU holds one big tile or two small ones; per 64-wide K stage a CU that is kept busy
-// needs about 2.0 us for a big tile and 0.78 us for a small one (measured in the model, weights
-// from HBM: about 1060 and 700 TFLOP/s; the wider a wave's own tile and the more waves share an
-// operand, the fewer LDS bytes per product).  What counts is the CU with the most tiles.  A
+// shape: 0 = choose, 1 = 128x128 tiles, 2 = 256x256, 3 = 256x192.  The choice is made on an
+// estimate of the time.  A CU holds one big tile or two small ones; per 64-wide K stage a CU
+// that is kept busy needs about 2.0 us for a 256x256 tile, 1.62 us for a 256x192 one and 0.78 us
+// for a small one (measured in the model, weights from HBM: about 1060, 980 and 700 TFLOP/s; the
+// wider a wave's own tile and the more waves share an operand, the fewer LDS bytes per product).
+// What counts is the CU with the most tiles: 6144 columns are 24 tiles of 256, which with 2048
+// rows leave a quarter of the chip idle, or 32 tiles of 192, which fill it.  A
 // product with few tiles (few rows, or a narrow output) leaves most CUs idle while a few walk
 // through all of K: then K is cut into up to 8 pieces, each the work of a block of its own,
 // at the price of writing and reading the 32-bit partial sums once more.  No estimate may go
@@ -71,10 +73,11 @@ static int launch_mfma_tile(const void* x, int ldx, const void* w, int ldw, void
     int splits = 1;
     if (shape == 0) {
         double best = 1e30;
-        for (int big = 0; big < 2; ++big) {
-            int edge = big ? 256 : 128;
-            double stage_us = big ? 2.0 : 0.78;
-            long long tiles = (long long)ceil_div(m, edge) * ceil_div(n, edge);
+        // rows and columns of a tile, microseconds per 64-wide K stage, the shape's number
+        static const struct { int bm, bn; double stage_us; int shape; } kinds[] = {
+            {128, 128, 0.78, 1}, {256, 256, 2.0, 2}, {256, 192, 1.62, 3}};
+        for (const auto& kind : kinds) {
+            long long tiles = (long long)ceil_div(m, kind.bm) * ceil_div(n, kind.bn);
             for (int pieces = 1; pieces <= 8; ++pieces) {
                 if (pieces > 1 && (EPI == EPI_SWIGLU || k / pieces < 512 || !workspace ||
                                    (long long)pieces * m * n * (long long)sizeof(float) > workspace_bytes))
@@ -82,14 +85,15 @@ static int launch_mfma_tile(const void* x, int ldx, const void* w, int ldw, void
                 long long blocks = tiles * pieces;
                 double per_cu = (double)ceil_div(blocks, 256);          // tiles of the busiest CU
                 double stages = (double)ceil_div(ceil_div(k, pieces), GM_BK);
-                double t = per_cu * stages * stage_us + 4.0;
+                double t = per_cu * stages * kind.stage_us + 4.0;
                 if (pieces > 1) t += (double)pieces * m * n * 8.0 / 4.0e6;   // partial sums out and in, 4 TB/s
                 double floor_us = (double)n * k * 2.0 / 5.5e6;               // the weights at 5.5 TB/s
                 if (t < floor_us) t = floor_us;
-                if (t < best) { best = t; shape = big ? 2 : 1; splits = pieces; }
+                if (t < best) { best = t; shape = kind.shape; splits = pieces; }
             }
         }
     }
+    if (shape == 3) return launch_mfma_tile_as<EPI, GemmTile192>(x, ldx, w, ldw, out, ldo, m, n, k, splits, workspace, plan, stream);
     if (shape == 2) return launch_mfma_tile_as<EPI, GemmTile256>(x, ldx, w, ldw, out, ldo, m, n, k, splits, workspace, plan, stream);
     return launch_mfma_tile_as<EPI, GemmTile128>(x, ldx, w, ldw, out, ldo, m, n, k, splits, workspace, plan, stream);
 }
@@ -260,7 +264,7 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
     ROCML_REQUIRE(ldx >= k && ldw >= k && ldo >= out_cols, "gemm: row strides (%d, %d, %d) below (K, K, N)",
                   ldx, ldw, ldo);
     ROCML_REQUIRE(!accumulate || out_dtype == ROCML_F32, "gemm: accumulation needs a 32-bit output");
-    ROCML_REQUIRE(algo >= ALGO_AUTO && algo <= ALGO_MFMA_TILE256, "gemm: unknown algorithm %d", algo);
+    ROCML_REQUIRE(algo >= ALGO_AUTO && algo <= ALGO_MFMA_TILE192, "gemm: unknown algorithm %d", algo);
     ROCML_REQUIRE(!defer || deferred_splits, "gemm: deferring needs a place to report the splits");
     if (m == 0) return 0;
     bool bf16_in = x_dtype == ROCML_BF16 && w_dtype == ROCML_BF16;
@@ -297,7 +301,8 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
         if (kpar) rc = BY_EPI(launch_kpar, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
         else if (skinny) rc = BY_EPI(launch_skinny_m, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
         else rc = BY_EPI(launch_mfma_tile, x, ldx, w, ldw, out, ldo, m, n, k,
-                         algo == ALGO_MFMA_TILE ? 1 : algo == ALGO_MFMA_TILE256 ? 2 : 0, workspace, workspace_bytes,
+                         algo == ALGO_MFMA_TILE ? 1 : algo == ALGO_MFMA_TILE256 ? 2 : algo == ALGO_MFMA_TILE192 ? 3 : 0,
+                         workspace, workspace_bytes,
                          plan, stream);
 #undef BY_EPI
         if (rc) return rc;

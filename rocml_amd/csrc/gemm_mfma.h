@@ -76,6 +76,7 @@ struct GemmTile {
 };
 using GemmTile128 = GemmTile<2, 2, 2, 2>;
 using GemmTile256 = GemmTile<2, 4, 4, 2>;       // eight waves (two per SIMD), 128x64 each
+using GemmTile192 = GemmTile<4, 2, 2, 3>;       // 256 rows x 192 columns, eight waves of 64x96
 
 // Accumulator element e of a lane: row 8*(e/4) + 4*(lane/32) + e%4, column lane%32.
 template <int EPI, typename T>
