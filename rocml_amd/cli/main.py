@@ -75,7 +75,12 @@ def cmd_generate(args) -> int:
         raise RocmlError("give --prompt-ids (token ids) or --prompt (text, with a tokenizer.json)")
     model = _load(args, args.ctx)
     params = sampling_from_args(args, model.entry.sampling if model.entry else None)
-    results = model.generate(prompts, params, max_new_tokens=args.n, stop_tokens=_parse_ids(args.stop_ids or ""))
+    profiler = _profiler(args.dtype) if args.profile else None
+    if profiler is not None:
+        with profiler:
+            results = model.generate(prompts, params, max_new_tokens=args.n, stop_tokens=_parse_ids(args.stop_ids or ""))
+    else:
+        results = model.generate(prompts, params, max_new_tokens=args.n, stop_tokens=_parse_ids(args.stop_ids or ""))
     for i, r in enumerate(results):
         if tok is not None and i == len(results) - 1 and args.prompt is not None:
             print(tok.decode(r.tokens))
@@ -85,7 +90,16 @@ def cmd_generate(args) -> int:
     print(f"prompt: {s.prompt_tokens} tokens in {s.prompt_seconds:.3f} s ({s.prompt_tok_s():.1f} tok/s); "
           f"generated: {s.generated_tokens} tokens in {s.decode_seconds:.3f} s ({s.decode_tok_s():.1f} tok/s)",
           file=sys.stderr)
+    if profiler is not None:
+        print(profiler.finish().to_human())
     return 0
+
+
+def _profiler(dtype: str):
+    """Per-operation timing with a roofline report (rocml-cli/src/cmd_generate.rs:46-48,140-141)."""
+    import torch
+    from ..profile import OpProfiler
+    return OpProfiler(torch.bfloat16 if dtype == "bfloat16" else torch.float32)
 
 
 def cmd_bench(args) -> int:
@@ -97,10 +111,19 @@ def cmd_bench(args) -> int:
     model = _load(args, ctx)
     rng = np.random.default_rng(0)
     prefill, decode = [], []
-    for _ in range(args.runs):
+    # Only the last run is profiled; it still counts for the medians, as in the reference
+    # (rocml-cli/src/cmd_bench.rs:129-141), though its steps run launch by launch.
+    want_profile = args.profile or args.profile_json is not None
+    report = None
+    for run in range(args.runs):
         prompts = [[int(t) for t in rng.integers(0, model.vocab_size, size=prompt_tokens)]
                    for _ in range(args.batch)]
-        model.generate(prompts, max_new_tokens=args.decode_tokens)
+        if want_profile and run + 1 == args.runs:
+            with _profiler(args.dtype) as profiler:
+                model.generate(prompts, max_new_tokens=args.decode_tokens)
+            report = profiler.finish()
+        else:
+            model.generate(prompts, max_new_tokens=args.decode_tokens)
         s = model.last_stats
         prefill.append(s.prompt_tok_s())
         decode.append(s.decode_tok_s())
@@ -113,6 +136,11 @@ def cmd_bench(args) -> int:
         print(f"{args.model} {args.dtype} batch {args.batch}: prefill {out['prefill_tok_s']:.1f} tok/s "
               f"({prompt_tokens} tokens), decode {out['decode_tok_s']:.1f} tok/s ({args.decode_tokens} tokens), "
               f"median of {args.runs}")
+    if report is not None and args.profile:
+        print(report.to_human())
+    if report is not None and args.profile_json is not None:
+        with open(args.profile_json, "w", encoding="utf-8") as f:
+            json.dump({"bench": out, "report": report.to_dict()}, f, indent=1)
     return 0
 
 
@@ -158,6 +186,7 @@ def build_parser() -> argparse.ArgumentParser:
     g.add_argument("--ctx", type=int, default=None, help="longest sequence the cache is sized for")
     g.add_argument("--stop-ids", default=None, help="token ids that end a sequence")
     g.add_argument("--weights-seed", type=int, default=0, help="seed of the random weights of a catalog model")
+    g.add_argument("--profile", action="store_true", help="time every operation and print a roofline report")
     _add_sampling_args(g)
     g.set_defaults(fn=cmd_generate)
     b = sub.add_parser("bench", help="measure prefill and decode speed")
@@ -168,6 +197,8 @@ def build_parser() -> argparse.ArgumentParser:
     b.add_argument("--depth", type=int, default=None, help="prompt of this many tokens, then decode")
     b.add_argument("--ctx", type=int, default=None)
     b.add_argument("--json", action="store_true")
+    b.add_argument("--profile", action="store_true", help="time every operation of the last run and print a roofline report")
+    b.add_argument("--profile-json", default=None, metavar="PATH", help="write that report as JSON (implies profiling)")
     b.set_defaults(fn=cmd_bench)
     m = sub.add_parser("models", help="list the catalog")
     m.set_defaults(fn=cmd_models)

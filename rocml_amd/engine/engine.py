@@ -19,6 +19,7 @@ import torch
 
 from ..cache import Cache
 from ..errors import ContextOverflowError, RocmlError
+from .. import profile
 from .batch import StepContext, StepEntry, pack_step
 from .model import DecoderModel
 from .workspace import Workspace
@@ -163,7 +164,9 @@ class Engine:
         def run(step: StepContext) -> Optional[torch.Tensor]:
             return self.model.forward(step, self.cache, step.block_tables, step.want_rows, n_want)
 
-        if not (self.use_graphs and max_new == 1 and len(slots) <= self.max_graph_batch):
+        profile.set_phase("decode" if max_new == 1 else "prefill")
+        # (a profiler times single launches: no recorded graph while one is active)
+        if not (self.use_graphs and max_new == 1 and len(slots) <= self.max_graph_batch) or profile.active() is not None:
             return run(context())
         # Decode steps of one shape run from a recorded graph: the launches of a step are the
         # same every time, only the integer tables change, and those lie at fixed addresses.

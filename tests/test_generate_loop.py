@@ -136,3 +136,28 @@ def test_rng_matches_the_reference_generator():
     assert sequence_seed(5, 0) == 5 and len({sequence_seed(5, i) for i in range(100)}) == 100
     assert SamplingParams().is_greedy() and not SamplingParams(temperature=0.7).is_greedy()
     assert not SamplingParams(repeat_penalty=1.0).penalty_active() and SamplingParams(repeat_penalty=1.1).penalty_active()
+
+
+def test_profile_report_rows_and_roofline_columns():
+    """The per-operation report from raw records: time share, rates, analytical minimum
+    t_min = max(bytes / bandwidth, flops / peak), efficiency and wasted time per row
+    (rocml/src/profile/report.rs:21-75), phases apart, worklist by wasted time."""
+    from rocml_amd.profile import HBM_BYTES_PER_S, build_report
+    peak = 2.5e15
+    records = [("decode", "product", 8_000_000_000, 1_000_000, 2.0),       # memory bound: t_min 1 ms
+               ("decode", "product", 8_000_000_000, 1_000_000, 2.0),
+               ("decode", "rmsnorm", 80_000, 0, 0.5),
+               ("prefill", "product", 1_000, 5_000_000_000_000, 4.0)]      # compute bound: t_min 2 ms
+    rep = build_report(records, peak)
+    assert [p.phase for p in rep.phases] == ["prefill", "decode"]
+    dec = rep.phases[1]
+    assert dec.total_elapsed_ms == 4.5 and [r.label for r in dec.by_op] == ["product", "rmsnorm"]
+    prod = dec.by_op[0]
+    assert prod.count == 2 and prod.bytes == 16_000_000_000
+    assert abs(prod.t_min_ms - 1e3 * 16e9 / HBM_BYTES_PER_S) < 1e-9 and abs(prod.efficiency - 0.5) < 1e-9
+    assert abs(prod.wasted_ms - 2.0) < 1e-9 and abs(prod.gb_per_sec - 4000.0) < 1e-6
+    assert abs(prod.pct_of_bandwidth_roofline - 50.0) < 1e-9 and abs(prod.pct_of_phase_time - 100 * 4 / 4.5) < 1e-9
+    pre = rep.phases[0].by_op[0]
+    assert abs(pre.t_min_ms - 2.0) < 1e-9 and abs(pre.pct_of_flop_roofline - 50.0) < 1e-9
+    assert rep.worklist[0].startswith("decode product") or rep.worklist[0].startswith("prefill product")
+    assert "t_min ms" in rep.to_human() and "report" in rep.to_json()

@@ -123,3 +123,33 @@ def test_command_line_generate_and_models(models, capsys):
     assert main(["models"]) == 0 and "qwen3-8b" in capsys.readouterr().out
     assert main(["generate", "--model", "no-such-model", "--prompt-ids", "1"]) == 1
     assert "known names" in capsys.readouterr().err
+
+
+def test_command_line_profile_report(models, capsys, tmp_path):
+    """--profile times every operation (steps then run launch by launch) and prints the report;
+    the tokens are those of an unprofiled run; bench --profile-json writes the report."""
+    import json
+    from rocml_amd.cli import main
+    path, cfg, weights = models["B"]
+    prompt = helpers.random_tokens(9, cfg["vocab_size"], 6)
+    argv = ["generate", "--model", path, "--dtype", "float32", "--prompt-ids", " ".join(map(str, prompt)),
+            "-n", "6", "--ctx", "64", "--batch", "2"]
+    assert main(argv) == 0
+    plain_out = capsys.readouterr().out.strip().splitlines()
+    assert main(argv + ["--profile"]) == 0
+    out = capsys.readouterr().out.strip().splitlines()
+    assert out[0] == plain_out[0] and [int(t) for t in out[0].split()] == plain.greedy(cfg, weights, prompt, 6)
+    text = "\n".join(out[1:])
+    assert text.startswith("prefill:") and "\ndecode:" in text
+    for label in ("product", "attention", "rmsnorm", "embedding", "argmax"):
+        assert label in text
+    report_path = tmp_path / "report.json"
+    assert main(["bench", "--model", path, "--dtype", "bfloat16", "--prompt-tokens", "20", "--decode-tokens", "4",
+                 "--runs", "2", "--batch", "2", "--ctx", "64", "--json", "--profile-json", str(report_path)]) == 0
+    doc = json.loads(report_path.read_text())
+    phases = {p["phase"]: p for p in doc["report"]["phases"]}
+    assert set(phases) == {"prefill", "decode"} and doc["bench"]["decode_tokens"] == 4
+    products = [r for r in phases["decode"]["by_op"] if r["label"] == "product"][0]
+    n_layers = cfg["num_hidden_layers"]
+    assert products["count"] == 3 * (4 * n_layers + 1)            # four products a layer and the output, three decode steps
+    assert products["elapsed_ms"] > 0 and products["t_min_ms"] > 0 and 0 < products["efficiency"]
