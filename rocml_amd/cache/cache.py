@@ -29,7 +29,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import numpy as np
 import torch
 
-from ..errors import CacheFullError, RocmlError
+from ..errors import CacheFullError, MemoryBudgetError, RocmlError
 from ..parts.base import KVCacheRequest, StateRequest
 
 PAGE_SIZE = 64
@@ -184,15 +184,61 @@ class CacheLineView:
     slots: Optional[torch.Tensor] = None        # [B] int32 on the device, per step
 
 
+# Memory left free beside the cache for activations and the runtime: the reference keeps
+# 768 MiB of headroom when it checks a context length against hipMemGetInfo
+# (rocml/src/budget/mod.rs:37, rocml/src/forward/mod.rs:148-161).
+HEADROOM_BYTES = 768 << 20
+
+
+def _group_pages(req: KVCacheRequest, n_pages: int, max_seqs: Optional[int], page_size: int) -> int:
+    """Pages of a key/value group: a windowed group never holds more than a window and a page
+    per sequence."""
+    if req.window is not None and max_seqs is not None:
+        return min(n_pages, max_seqs * (pages_for(req.window, page_size) + 1))
+    return n_pages
+
+
+def planned_bytes(requests: Sequence[Optional[object]], max_tokens: int, dtype: torch.dtype,
+                  max_seqs: Optional[int] = None, page_size: int = PAGE_SIZE) -> int:
+    """Bytes the cache for these requests will allocate: per key/value line
+    ``2 * pages * page_size * Hkv * D * bytes`` (rocml/src/budget/mod.rs:47-59), per state
+    line ``slots * elements * bytes``."""
+    n_pages = max(1, pages_for(max_tokens, page_size))
+    slots = max_seqs if max_seqs is not None else n_pages
+    size = torch.empty((), dtype=dtype).element_size()
+    total = 0
+    for req in requests:
+        if isinstance(req, KVCacheRequest):
+            total += 2 * _group_pages(req, n_pages, max_seqs, page_size) * page_size * req.n_kv_heads * req.head_dim * size
+        elif isinstance(req, StateRequest):
+            n = 1
+            for dim in req.shape:
+                n *= dim
+            total += slots * n * torch.empty((), dtype=req.dtype).element_size()
+    return total
+
+
+def check_budget(need: int, free: int, headroom: int = HEADROOM_BYTES) -> None:
+    if need + headroom > free:
+        raise MemoryBudgetError(
+            f"the cache needs {need / 2**30:.2f} GiB and {headroom / 2**20:.0f} MiB are kept free beside it, but the "
+            f"device has {free / 2**30:.2f} GiB free: ask for fewer positions or sequences")
+
+
 class Cache:
     """Slots, groups and the mapping from schedule entries to cache lines.
 
     ``requests[i]`` is what schedule entry ``i`` asks for (``None`` for an entry that
     owns no cache line).  ``max_tokens`` is the number of positions live sequences may
-    hold together, each rounded up to whole pages; ``max_seqs`` bounds the live sequences."""
+    hold together, each rounded up to whole pages; ``max_seqs`` bounds the live sequences.
+    With ``free_bytes`` (the free memory of the device) the storage is checked against it
+    before anything is allocated."""
 
     def __init__(self, requests: Sequence[Optional[object]], max_tokens: int, dtype: torch.dtype,
-                 device, max_seqs: Optional[int] = None, page_size: int = PAGE_SIZE):
+                 device, max_seqs: Optional[int] = None, page_size: int = PAGE_SIZE,
+                 free_bytes: Optional[int] = None):
+        if free_bytes is not None:
+            check_budget(planned_bytes(requests, max_tokens, dtype, max_seqs, page_size), free_bytes)
         self.page_size = page_size
         self.n_pages = max(1, pages_for(max_tokens, page_size))
         self.max_seqs = max_seqs if max_seqs is not None else self.n_pages
@@ -207,9 +253,7 @@ class Cache:
                 by_request.setdefault(req, []).append(entry)
         for req, entries in by_request.items():
             if isinstance(req, KVCacheRequest):
-                n_pages = self.n_pages
-                if req.window is not None and max_seqs is not None:
-                    n_pages = min(n_pages, max_seqs * (pages_for(req.window, page_size) + 1))
+                n_pages = _group_pages(req, self.n_pages, max_seqs, page_size)
                 name = f"kv{len(self.kv_groups)}" + ("" if req.window is None else f"w{req.window}")
                 group = KVGroup(name, req, len(entries), n_pages, page_size, dtype, device)
                 self.kv_groups.append(group)

@@ -81,7 +81,12 @@ class DecoderModel:
                 for e in self.spec.schedule]
 
     def new_cache(self, max_tokens: int, max_seqs: Optional[int] = None) -> Cache:
-        return Cache(self.cache_requests(), max_tokens, self.dtype, self.device, max_seqs=max_seqs)
+        free = None
+        if torch.device(self.device).type == "cuda":
+            # what the driver reports as free, and what torch holds without using it
+            free = torch.cuda.mem_get_info(self.device)[0] + \
+                torch.cuda.memory_reserved(self.device) - torch.cuda.memory_allocated(self.device)
+        return Cache(self.cache_requests(), max_tokens, self.dtype, self.device, max_seqs=max_seqs, free_bytes=free)
 
     # -- forward -----------------------------------------------------------------------
     def forward(self, step: StepContext, cache: Cache, block_tables: Dict[str, torch.Tensor],

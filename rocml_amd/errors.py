@@ -31,6 +31,10 @@ class CacheFullError(RocmlError):
     """The cache cannot hold the tokens or sequences a step asks for."""
 
 
+class MemoryBudgetError(RocmlError):
+    """The cache that was asked for does not fit the free memory of the GPU."""
+
+
 class ContextOverflowError(RocmlError):
     """A sequence would grow beyond the positions the model was built for."""
 

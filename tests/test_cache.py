@@ -145,3 +145,25 @@ def test_random_traffic_keeps_the_books_balanced():
                 assert all(p >= 0 for p in table[first:])          # every page a query may read is held
     held = [p for g in c.kv_groups[:1] for s in live for p in g.page_table(s) if p >= 0]
     assert len(held) == len(set(held))                              # no page held twice
+
+
+def test_storage_is_checked_against_free_memory_before_it_is_allocated():
+    """Bytes per position as the reference counts them (2 * lines * Hkv * D * bytes,
+    rocml/src/budget/mod.rs:47-59), 768 MiB kept free beside the cache, and a refusal that
+    allocates nothing."""
+    from rocml_amd.cache.cache import HEADROOM_BYTES, check_budget, planned_bytes
+    from rocml_amd.errors import MemoryBudgetError
+    full = KVCacheRequest(n_kv_heads=8, head_dim=128, window=None)
+    windowed = KVCacheRequest(n_kv_heads=2, head_dim=64, window=100)
+    state = StateRequest(shape=(4, 16), dtype=torch.float32)
+    need = planned_bytes([full, full, None, windowed, state], max_tokens=64 * 1000, dtype=torch.bfloat16, max_seqs=10)
+    kv_full = 2 * 2 * 64 * 1000 * 8 * 128 * 2                       # two lines of 1000 pages
+    kv_window = 2 * (10 * 3) * 64 * 2 * 64 * 2                      # a window of 100 is two pages and one more, per sequence
+    assert need == kv_full + kv_window + 10 * 64 * 4
+    check_budget(need, need + HEADROOM_BYTES)
+    with pytest.raises(MemoryBudgetError, match="GiB free"):
+        check_budget(need, need + HEADROOM_BYTES - 1)
+    with pytest.raises(MemoryBudgetError):
+        Cache([full], max_tokens=1 << 40, dtype=torch.bfloat16, device="cpu", free_bytes=1 << 30)
+    cache = Cache([full], max_tokens=128, dtype=torch.float32, device="cpu", free_bytes=HEADROOM_BYTES + (1 << 20))
+    assert cache.n_pages == 2
