@@ -218,11 +218,16 @@ def planned_bytes(requests: Sequence[Optional[object]], max_tokens: int, dtype: 
     return total
 
 
-def check_budget(need: int, free: int, headroom: int = HEADROOM_BYTES) -> None:
+def check_budget(need: int, free: int, headroom: int = HEADROOM_BYTES, max_tokens: Optional[int] = None) -> None:
+    """Raises when ``need`` bytes and the headroom do not fit ``free``; names, as the reference's
+    budget does (rocml/src/budget/mod.rs:70-83), about how many positions would fit."""
     if need + headroom > free:
+        hint = ""
+        if max_tokens is not None and need > 0:
+            hint = f" (about {max(0, free - headroom) * max_tokens // need} positions would fit)"
         raise MemoryBudgetError(
             f"the cache needs {need / 2**30:.2f} GiB and {headroom / 2**20:.0f} MiB are kept free beside it, but the "
-            f"device has {free / 2**30:.2f} GiB free: ask for fewer positions or sequences")
+            f"device has {free / 2**30:.2f} GiB free: ask for fewer positions or sequences{hint}")
 
 
 class Cache:
@@ -238,7 +243,7 @@ class Cache:
                  device, max_seqs: Optional[int] = None, page_size: int = PAGE_SIZE,
                  free_bytes: Optional[int] = None):
         if free_bytes is not None:
-            check_budget(planned_bytes(requests, max_tokens, dtype, max_seqs, page_size), free_bytes)
+            check_budget(planned_bytes(requests, max_tokens, dtype, max_seqs, page_size), free_bytes, max_tokens=max_tokens)
         self.page_size = page_size
         self.n_pages = max(1, pages_for(max_tokens, page_size))
         self.max_seqs = max_seqs if max_seqs is not None else self.n_pages
