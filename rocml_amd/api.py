@@ -85,6 +85,18 @@ class Model:
     def step(self, entries: Sequence[StepEntry]):
         return self.engine.step(entries)
 
+    def position(self, slot: int) -> int:
+        """Tokens the sequence holds so far (the reference's ``position()``,
+        rocml/src/model.rs:112-130, per sequence here)."""
+        return self.engine.length(slot)
+
+    def reset(self) -> None:
+        """Ends every live sequence; their slots and pages are given back and nothing is
+        cleared, as rows beyond a length are never read (the reference's ``reset()`` sets
+        its one position to zero, rocml/src/forward/mod.rs:224-232)."""
+        for slot in sorted(self.engine.cache.slots.live):
+            self.engine.release(slot)
+
     # -- generation ----------------------------------------------------------------------
     def generate(self, prompts: Sequence[Sequence[int]],
                  sampling: Union[SamplingParams, Sequence[SamplingParams], None] = None,

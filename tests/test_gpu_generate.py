@@ -153,3 +153,20 @@ def test_command_line_profile_report(models, capsys, tmp_path):
     n_layers = cfg["num_hidden_layers"]
     assert products["count"] == 3 * (4 * n_layers + 1)            # four products a layer and the output, three decode steps
     assert products["elapsed_ms"] > 0 and products["t_min_ms"] > 0 and 0 < products["efficiency"]
+
+
+def test_position_and_reset_through_the_entry_point(models):
+    from rocml_amd.engine import StepEntry
+    path, cfg, weights = models["A"]
+    model = _load(path, "float32", ctx=64, max_batch=2)
+    toks = helpers.random_tokens(20, cfg["vocab_size"], 3)
+    ref = plain.forward(cfg, weights, toks)
+    a, b = model.new_sequence(), model.new_sequence()
+    model.step([StepEntry(a, toks[:7], []), StepEntry(b, toks[:3], [])])
+    assert model.position(a) == 7 and model.position(b) == 3
+    model.reset()
+    model.engine.cache.check()
+    assert not model.engine.cache.lengths
+    c = model.new_sequence()                       # a slot and pages that were just given back, not cleared
+    got = model.step([StepEntry(c, toks, list(range(20)))]).cpu()
+    assert model.position(c) == 20 and helpers.rel_to_max(got, ref) < 2e-5
