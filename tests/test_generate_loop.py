@@ -161,3 +161,19 @@ def test_profile_report_rows_and_roofline_columns():
     assert abs(pre.t_min_ms - 2.0) < 1e-9 and abs(pre.pct_of_flop_roofline - 50.0) < 1e-9
     assert rep.worklist[0].startswith("decode product") or rep.worklist[0].startswith("prefill product")
     assert "t_min ms" in rep.to_human() and "report" in rep.to_json()
+
+
+def test_profiler_wraps_the_launch_helpers_only_while_it_is_active():
+    import torch
+    from rocml_amd import ops, profile
+    before = {name: getattr(ops, name) for name in ("gemm", "rmsnorm", "attention", "sample")}
+    assert profile.active() is None
+    with profile.OpProfiler(torch.float32) as p:
+        assert profile.active() is p and ops.gemm is not before["gemm"]
+        profile.set_phase("decode")
+        assert p.phase == "decode"
+        with pytest.raises(RuntimeError):
+            profile.OpProfiler().__enter__()
+    assert profile.active() is None
+    assert all(getattr(ops, name) is fn for name, fn in before.items())
+    profile.set_phase("prefill")                     # without a profiler: nothing to tag
