@@ -32,6 +32,26 @@ class LoadOptions:
     use_graphs: bool = True
 
 
+def _generation_config_eos(path: str, vocab: int) -> frozenset:
+    import json
+    import os
+    file = os.path.join(path, "generation_config.json")
+    if not os.path.isfile(file):
+        return frozenset()
+    try:
+        with open(file, "r", encoding="utf-8") as f:
+            eos = json.load(f).get("eos_token_id")
+    except (OSError, ValueError) as e:
+        raise RocmlError(f"{file} cannot be read: {e}") from e
+    if eos is None:
+        return frozenset()
+    ids = eos if isinstance(eos, (list, tuple)) else [eos]
+    for t in ids:
+        if isinstance(t, bool) or not isinstance(t, int) or not 0 <= t < vocab:
+            raise RocmlError(f"{file}: eos_token_id must name token ids below {vocab}, found {eos!r}")
+    return frozenset(ids)
+
+
 class Model:
     """A loaded model with its engine."""
 
@@ -40,6 +60,10 @@ class Model:
         self.options = options
         self.entry = entry
         self.last_stats: Optional[GenerateStats] = None
+        # ids that end a sequence by default: config.json's, and generation_config.json's if the
+        # folder has one (the reference takes the id from its checkpoint and stops there unless
+        # told not to, rocml/src/generate/resumed.rs:170,217-219)
+        self.eos_token_ids = frozenset(engine.model.spec.eos_token_ids)
 
     @staticmethod
     def load(name_or_path: str, options: Optional[LoadOptions] = None, **kwargs) -> "Model":
@@ -58,7 +82,10 @@ class Model:
         max_tokens = options.max_tokens or ctx * options.max_batch
         engine = Engine(model, max_tokens=max_tokens, max_seqs=max(options.max_batch, 1),
                         use_graphs=options.use_graphs)
-        return Model(engine, options, found.entry)
+        loaded = Model(engine, options, found.entry)
+        if found.path is not None:
+            loaded.eos_token_ids |= _generation_config_eos(found.path, model.spec.vocab)
+        return loaded
 
     @property
     def config(self):
@@ -100,10 +127,12 @@ class Model:
     # -- generation ----------------------------------------------------------------------
     def generate(self, prompts: Sequence[Sequence[int]],
                  sampling: Union[SamplingParams, Sequence[SamplingParams], None] = None,
-                 max_new_tokens: int = 64, stop_tokens: Iterable[int] = ()) -> List[Result]:
+                 max_new_tokens: int = 64, stop_tokens: Iterable[int] = (), ignore_eos: bool = False,
+                 on_step=None) -> List[Result]:
         """Continues every prompt (lists of token ids).  ``sampling`` is one set of parameters
         for all prompts or one per prompt; ``None`` means greedy.  A stop token ends its
-        sequence and is not part of the result."""
+        sequence and is not part of the result; the model's end-of-sequence ids are stop tokens
+        unless ``ignore_eos``.  ``on_step`` is called after every decode step with their number."""
         if sampling is None:
             sampling = SamplingParams.greedy()
         if isinstance(sampling, SamplingParams):
@@ -111,8 +140,11 @@ class Model:
         if len(sampling) != len(prompts):
             raise RocmlError("one SamplingParams for all prompts, or one per prompt")
         stop = frozenset(int(t) for t in stop_tokens)
+        if not ignore_eos:
+            stop |= self.eos_token_ids
         requests = [Request(list(p), max_new_tokens, s, stop) for p, s in zip(prompts, sampling)]
         gen = Generator(EngineBackend(self.engine), max_batch=self.options.max_batch)
+        gen.on_step = on_step
         results = gen.run(requests)
         self.last_stats = gen.stats
         return results

@@ -190,16 +190,22 @@ class CacheLineView:
 HEADROOM_BYTES = 768 << 20
 
 
-def _group_pages(req: KVCacheRequest, n_pages: int, max_seqs: Optional[int], page_size: int) -> int:
-    """Pages of a key/value group: a windowed group never holds more than a window and a page
-    per sequence."""
-    if req.window is not None and max_seqs is not None:
-        return min(n_pages, max_seqs * (pages_for(req.window, page_size) + 1))
+def _group_pages(req: KVCacheRequest, n_pages: int, max_seqs: Optional[int], page_size: int,
+                 step_tokens: Optional[int] = None) -> int:
+    """Pages of a key/value group.  A group with a window holds, per sequence, the pages its
+    window spans (one more than the window's pages, as it rarely starts on a page's edge) and
+    the page being filled; while a step runs it also holds the pages of the step's own tokens,
+    which are only given back when the step's piece is committed.  With a bound on the
+    sequences and on the tokens of a piece the group needs no more than that, however long
+    the sequences grow; without them it is sized like a group that keeps everything."""
+    if req.window is not None and max_seqs is not None and step_tokens is not None:
+        return min(n_pages, max_seqs * (pages_for(req.window, page_size) + 2) + pages_for(step_tokens, page_size))
     return n_pages
 
 
 def planned_bytes(requests: Sequence[Optional[object]], max_tokens: int, dtype: torch.dtype,
-                  max_seqs: Optional[int] = None, page_size: int = PAGE_SIZE) -> int:
+                  max_seqs: Optional[int] = None, page_size: int = PAGE_SIZE,
+                  step_tokens: Optional[int] = None) -> int:
     """Bytes the cache for these requests will allocate: per key/value line
     ``2 * pages * page_size * Hkv * D * bytes`` (rocml/src/budget/mod.rs:47-59), per state
     line ``slots * elements * bytes``."""
@@ -209,7 +215,7 @@ def planned_bytes(requests: Sequence[Optional[object]], max_tokens: int, dtype: 
     total = 0
     for req in requests:
         if isinstance(req, KVCacheRequest):
-            total += 2 * _group_pages(req, n_pages, max_seqs, page_size) * page_size * req.n_kv_heads * req.head_dim * size
+            total += 2 * _group_pages(req, n_pages, max_seqs, page_size, step_tokens) * page_size * req.n_kv_heads * req.head_dim * size
         elif isinstance(req, StateRequest):
             n = 1
             for dim in req.shape:
@@ -236,14 +242,18 @@ class Cache:
     ``requests[i]`` is what schedule entry ``i`` asks for (``None`` for an entry that
     owns no cache line).  ``max_tokens`` is the number of positions live sequences may
     hold together, each rounded up to whole pages; ``max_seqs`` bounds the live sequences.
-    With ``free_bytes`` (the free memory of the device) the storage is checked against it
-    before anything is allocated."""
+    ``step_tokens`` is the most tokens one piece of a step brings; with it and ``max_seqs`` a
+    group with a window is sized for its windows instead of for whole sequences.
+    With ``free_bytes`` (the free memory of the device) the storage is checked against it,
+    less ``headroom`` bytes for activations and the runtime, before anything is allocated."""
 
     def __init__(self, requests: Sequence[Optional[object]], max_tokens: int, dtype: torch.dtype,
                  device, max_seqs: Optional[int] = None, page_size: int = PAGE_SIZE,
-                 free_bytes: Optional[int] = None):
+                 free_bytes: Optional[int] = None, step_tokens: Optional[int] = None,
+                 headroom: int = HEADROOM_BYTES):
         if free_bytes is not None:
-            check_budget(planned_bytes(requests, max_tokens, dtype, max_seqs, page_size), free_bytes, max_tokens=max_tokens)
+            check_budget(planned_bytes(requests, max_tokens, dtype, max_seqs, page_size, step_tokens), free_bytes,
+                         headroom=headroom, max_tokens=max_tokens)
         self.page_size = page_size
         self.n_pages = max(1, pages_for(max_tokens, page_size))
         self.max_seqs = max_seqs if max_seqs is not None else self.n_pages
@@ -258,7 +268,7 @@ class Cache:
                 by_request.setdefault(req, []).append(entry)
         for req, entries in by_request.items():
             if isinstance(req, KVCacheRequest):
-                n_pages = _group_pages(req, self.n_pages, max_seqs, page_size)
+                n_pages = _group_pages(req, self.n_pages, max_seqs, page_size, step_tokens)
                 name = f"kv{len(self.kv_groups)}" + ("" if req.window is None else f"w{req.window}")
                 group = KVGroup(name, req, len(entries), n_pages, page_size, dtype, device)
                 self.kv_groups.append(group)
@@ -299,6 +309,54 @@ class Cache:
                     f"positions, {g.n_free_pages} of {g.n_pages} are free")
         for g in self.kv_groups:
             g.grow_together(slots, new_lens)
+
+    def fits(self, pieces: Sequence[Sequence[Tuple[object, int]]],
+             final: Optional[Sequence[Tuple[object, int]]] = None) -> Optional[str]:
+        """Whether the pieces of a step can be reserved and committed one after the other.
+        A piece is a list of ``(sequence, length after the piece)``; a sequence is a live slot
+        or any other key, which stands for a sequence that would start empty.  ``final`` names
+        the lengths the sequences will grow to afterwards, a token at a time.  Only page counts
+        are followed, nothing changes.  Returns None when everything fits, else what is short."""
+        for g in self.kv_groups:
+            free = g.n_free_pages
+            size: Dict[object, int] = {}
+            released: Dict[object, int] = {}
+            w = g.request.window
+            for piece in pieces:
+                need = 0
+                for key, n in piece:
+                    if key not in size:
+                        table = g._pages.get(key, []) if isinstance(key, int) else []
+                        size[key] = len(table)
+                        released[key] = sum(1 for p in table if p < 0)
+                    want = pages_for(n, g.page_size)
+                    if want > size[key]:
+                        need += want - size[key]
+                        size[key] = want
+                if need > free:
+                    return (f"cache group {g.name}: the step needs {need} more pages of {g.page_size} "
+                            f"positions, {free} of {g.n_pages} are free")
+                free -= need
+                if w is not None:        # what the commit of this piece gives back
+                    for key, n in piece:
+                        first_needed = min(max(0, n - w + 1) // g.page_size, size[key])
+                        if first_needed > released[key]:
+                            free += first_needed - released[key]
+                            released[key] = first_needed
+            if final:
+                # a token at a time: a sequence of a windowed group then never holds more than
+                # the pages its window spans and the one being filled
+                need = 0
+                for key, n in final:
+                    held = size.get(key, 0) - released.get(key, 0)
+                    want = pages_for(n, g.page_size) - released.get(key, 0)
+                    if w is not None:
+                        want = min(want, max(held, pages_for(w, g.page_size) + 2))
+                    need += max(0, want - held)
+                if need > free:
+                    return (f"cache group {g.name}: the sequences would need {need} more pages of "
+                            f"{g.page_size} positions, {free} of {g.n_pages} are free")
+        return None
 
     def commit(self, slots: Sequence[int], new_lens: Sequence[int]) -> None:
         for s, n in zip(slots, new_lens):

@@ -76,11 +76,12 @@ def cmd_generate(args) -> int:
     model = _load(args, args.ctx)
     params = sampling_from_args(args, model.entry.sampling if model.entry else None)
     profiler = _profiler(args.dtype) if args.profile else None
+    kwargs = dict(max_new_tokens=args.n, stop_tokens=_parse_ids(args.stop_ids or ""), ignore_eos=args.ignore_eos)
     if profiler is not None:
         with profiler:
-            results = model.generate(prompts, params, max_new_tokens=args.n, stop_tokens=_parse_ids(args.stop_ids or ""))
+            results = model.generate(prompts, params, **kwargs)
     else:
-        results = model.generate(prompts, params, max_new_tokens=args.n, stop_tokens=_parse_ids(args.stop_ids or ""))
+        results = model.generate(prompts, params, **kwargs)
     for i, r in enumerate(results):
         if tok is not None and i == len(results) - 1 and args.prompt is not None:
             print(tok.decode(r.tokens))
@@ -185,6 +186,8 @@ def build_parser() -> argparse.ArgumentParser:
     g.add_argument("-n", "--max-tokens", dest="n", type=int, default=64)
     g.add_argument("--ctx", type=int, default=None, help="longest sequence the cache is sized for")
     g.add_argument("--stop-ids", default=None, help="token ids that end a sequence")
+    g.add_argument("--ignore-eos", action="store_true",
+                   help="do not stop at the model's end-of-sequence id (eos_token_id of config.json or generation_config.json)")
     g.add_argument("--weights-seed", type=int, default=0, help="seed of the random weights of a catalog model")
     g.add_argument("--profile", action="store_true", help="time every operation and print a roofline report")
     _add_sampling_args(g)

@@ -43,6 +43,7 @@ class Qwen3Config:
     hidden_act: str = "silu"
     sliding_window: Optional[int] = None
     layer_types: Optional[Tuple[str, ...]] = None
+    eos_token_id: Optional[Tuple[int, ...]] = None
     architectures: Tuple[str, ...] = field(default=(ARCHITECTURE,))
 
     # ---- reading ---------------------------------------------------------
@@ -87,6 +88,14 @@ class Qwen3Config:
             values["layer_types"] = tuple(layer_types)
             if any(t == "sliding_attention" for t in layer_types):
                 values["sliding_window"] = window
+        eos = raw.get("eos_token_id")
+        if eos is not None:
+            # one id or a list of them; generation stops at any of them
+            ids = list(eos) if isinstance(eos, (list, tuple)) else [eos]
+            for t in ids:
+                if isinstance(t, bool) or not isinstance(t, int) or not 0 <= t < values["vocab_size"]:
+                    raise ConfigError(f"config.json key 'eos_token_id' must name token ids below vocab_size, found {eos!r}")
+            values["eos_token_id"] = tuple(ids)
         cfg = cls(**values)
         cfg.validate()
         return cfg
@@ -112,6 +121,16 @@ class Qwen3Config:
             d.pop("sliding_window")
         else:
             d["layer_types"] = list(self.layer_types)
+            # the older pair of keys that says the same for files read by the boundary: layers
+            # from max_window_layers on slide (when the sliding layers are the trailing ones)
+            sliding = [t == "sliding_attention" for t in self.layer_types]
+            d["use_sliding_window"] = any(sliding)
+            if any(sliding) and sliding == sorted(sliding):
+                d["max_window_layers"] = sliding.index(True)
+        if self.eos_token_id is None:
+            d.pop("eos_token_id")
+        else:
+            d["eos_token_id"] = list(self.eos_token_id) if len(self.eos_token_id) > 1 else self.eos_token_id[0]
         return d
 
     # ---- rules -----------------------------------------------------------
@@ -185,7 +204,8 @@ class Qwen3Config:
         spec = ModelSpec(architecture=ARCHITECTURE, vocab=self.vocab_size, hidden=self.hidden_size,
                          layers=tuple(layers), schedule=default_schedule(self.num_hidden_layers),
                          final_norm=hidden_norm, tie_lm_head=self.tie_word_embeddings,
-                         max_positions=self.max_position_embeddings)
+                         max_positions=self.max_position_embeddings,
+                         eos_token_ids=self.eos_token_id or ())
         spec.validate()
         return spec
 

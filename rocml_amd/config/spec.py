@@ -97,6 +97,7 @@ class ModelSpec:
     tie_lm_head: bool
     max_positions: int
     embed_scale: float = 1.0
+    eos_token_ids: Tuple[int, ...] = ()     # generation stops at any of these unless told otherwise
 
     def validate(self) -> None:
         from ..errors import ConfigError

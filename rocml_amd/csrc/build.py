@@ -4,12 +4,15 @@ The reference compiles every kernel source at build time with ``hipcc --genco
 --offload-arch=... -O3`` and fails with the compiler's output
 (rocml-kernels/build.rs:10-59).  Here each family (``elementwise``, ``gemm``,
 ``attention``, ``sampling``) becomes ``_build/lib<family>.so`` next to the sources;
-a family is compiled when it is first needed and no library is there yet, so a
-fresh checkout works without a build step.  ``python -m rocml_amd.csrc.build``
+a family is compiled when it is first needed and no library built from the present
+sources is there (a hash of the sources and flags is kept beside each library), so a
+fresh checkout works without a build step and an edited kernel is never run from an
+old library.  ``python -m rocml_amd.csrc.build``
 compiles all of them again.
 """
 from __future__ import annotations
 
+import hashlib
 import os
 import shutil
 import subprocess
@@ -54,7 +57,7 @@ def build_dir() -> str:
     """``_build`` beside the sources, or a per-user folder under the temporary
     directory when the checkout cannot be written."""
     local = os.path.join(SRC_DIR, "_build")
-    if os.path.isdir(local) and all(os.path.exists(os.path.join(local, f"lib{f}.so")) for f in FAMILIES):
+    if os.path.isdir(local) and all(is_current(os.path.join(local, f"lib{f}.so"), f) for f in FAMILIES):
         return local
     if _writable_dir(local):
         return local
@@ -64,9 +67,29 @@ def build_dir() -> str:
     raise ExtensionMissingError(f"neither {local} nor {alt} can be written")
 
 
+def source_hash(family: str) -> str:
+    """Hash of what a family's library is made from: its source, every header of the folder
+    (they are few, and any may be included) and the compiler flags."""
+    h = hashlib.sha256(" ".join([ARCH, *FLAGS]).encode())
+    names = [f"{family}.hip"] + sorted(n for n in os.listdir(SRC_DIR) if n.endswith(".h"))
+    for name in names:
+        with open(os.path.join(SRC_DIR, name), "rb") as f:
+            h.update(name.encode() + b"\0" + f.read() + b"\0")
+    return h.hexdigest()
+
+
+def is_current(path: str, family: str) -> bool:
+    """Whether ``path`` exists and was built from the present sources."""
+    try:
+        with open(path + ".srchash", "r", encoding="utf-8") as f:
+            return os.path.exists(path) and f.read().strip() == source_hash(family)
+    except OSError:
+        return False
+
+
 def library_path(family: str) -> str:
     local = os.path.join(SRC_DIR, "_build", f"lib{family}.so")
-    if os.path.exists(local):
+    if is_current(local, family):
         return local
     return os.path.join(build_dir(), f"lib{family}.so")
 
@@ -89,11 +112,13 @@ def _compile(family: str, out_path: str, log: List[str]) -> None:
         log.append(f"hipcc failed for {family}.hip:\n{output}")
         return
     os.replace(tmp, out_path)
+    with open(out_path + ".srchash", "w", encoding="utf-8") as f:
+        f.write(source_hash(family))
 
 
 def build(families: Iterable[str] = FAMILIES, force: bool = True, quiet: bool = False) -> Dict[str, str]:
     """Compiles the named families (in parallel) and returns their library paths.
-    With ``force=False`` a family whose library exists is left alone.  Prints a line
+    With ``force=False`` a family whose library was built from the present sources is left alone.  Prints a line
     when it starts, every few seconds while the compiler runs, and when it ends."""
     with _lock:
         out_dir = build_dir() if not force else (
@@ -105,7 +130,7 @@ def build(families: Iterable[str] = FAMILIES, force: bool = True, quiet: bool = 
                 raise ExtensionMissingError(f"unknown kernel family {fam!r}")
             path = os.path.join(out_dir, f"lib{fam}.so")
             paths[fam] = path
-            if force or not os.path.exists(path):
+            if force or not is_current(path, fam):
                 todo.append(fam)
         if not todo:
             return paths
@@ -134,9 +159,10 @@ def build(families: Iterable[str] = FAMILIES, force: bool = True, quiet: bool = 
 
 
 def ensure(family: str) -> str:
-    """Path of a family's library, compiling it first if it does not exist."""
+    """Path of a family's library, compiling it first if it does not exist or is older than
+    its sources."""
     path = library_path(family)
-    if os.path.exists(path):
+    if is_current(path, family):
         return path
     return build([family], force=False)[family]
 

@@ -18,7 +18,7 @@ import numpy as np
 import torch
 
 from ..cache import Cache
-from ..errors import ContextOverflowError, RocmlError
+from ..errors import CacheFullError, ContextOverflowError, RocmlError
 from .. import profile
 from .batch import StepContext, StepEntry, pack_step
 from .model import DecoderModel
@@ -38,9 +38,11 @@ class Engine:
         if model.embed is None:
             raise RocmlError("the model has no weights bound")
         self.model = model
-        self.cache: Cache = model.new_cache(max_tokens, max_seqs)
-        self.workspace = Workspace(model.device)
+        if max_step_tokens < 1:
+            raise RocmlError("max_step_tokens must be at least 1")
         self.max_step_tokens = max_step_tokens
+        self.cache: Cache = model.new_cache(max_tokens, max_seqs, step_tokens=max_step_tokens)
+        self.workspace = Workspace(model.device)
         self.steps_run = 0
         self.use_graphs = use_graphs
         self.max_graph_batch = 256
@@ -88,46 +90,64 @@ class Engine:
                     f"{spec.max_positions}")
             starts.append(start)
             new_lens.append(start + len(e.tokens))
-        self.cache.reserve(slots, new_lens)
-
-        total = sum(len(e.tokens) for e in entries)
+        # The step as pieces of at most max_step_tokens tokens (a sequence may straddle pieces).
+        # Pages are reserved piece by piece, and a piece is committed before the next runs, so a
+        # group with a window gives pages back while a long prompt passes through it; the whole
+        # plan is checked against the free pages first, so a step runs entirely or not at all.
+        pieces = self.plan_pieces([len(e.tokens) for e in entries])
+        short = self.cache.fits([[(entries[i].slot, starts[i] + hi) for i, _, hi in piece] for piece in pieces])
+        if short is not None:
+            raise CacheFullError(short)
         n_want_total = sum(len(e.want) for e in entries)
-        if total <= self.max_step_tokens:
+        if len(pieces) == 1:
+            self.cache.reserve(slots, new_lens)
             logits = self._run_piece(slots, starts, [list(e.tokens) for e in entries],
                                      [list(e.want) for e in entries])
             self.cache.commit(slots, new_lens)
             self.steps_run += 1
             return logits
 
-        # Cut the packed tokens into pieces; a sequence may straddle pieces.
         result = None
         if n_want_total:
             result = torch.empty((n_want_total, spec.vocab), dtype=torch.float32, device=self.model.device)
         want_base = np.cumsum([0] + [len(e.want) for e in entries])
-        done = [0] * len(entries)
-        while any(done[i] < len(e.tokens) for i, e in enumerate(entries)):
-            room = self.max_step_tokens
+        for piece in pieces:
             p_slots, p_starts, p_tokens, p_want, p_dest = [], [], [], [], []
-            for i, e in enumerate(entries):
-                left = len(e.tokens) - done[i]
-                if left == 0 or room == 0:
-                    continue
-                take = min(left, room)
-                lo, hi = done[i], done[i] + take
+            for i, lo, hi in piece:
+                e = entries[i]
                 wanted = [(k, w - lo) for k, w in enumerate(e.want) if lo <= w < hi]
                 p_slots.append(e.slot)
                 p_starts.append(starts[i] + lo)
                 p_tokens.append(list(e.tokens[lo:hi]))
                 p_want.append([w for _, w in wanted])
                 p_dest.extend(int(want_base[i]) + k for k, _ in wanted)
-                done[i] = hi
-                room -= take
+            p_lens = [s + len(t) for s, t in zip(p_starts, p_tokens)]
+            self.cache.reserve(p_slots, p_lens)
             logits = self._run_piece(p_slots, p_starts, p_tokens, p_want)
             if logits is not None:
                 result[torch.as_tensor(p_dest, device=self.model.device)] = logits
-            self.cache.commit(p_slots, [s + len(t) for s, t in zip(p_starts, p_tokens)])
+            self.cache.commit(p_slots, p_lens)
         self.steps_run += 1
         return result
+
+    def plan_pieces(self, counts: Sequence[int]) -> List[List[tuple]]:
+        """How a step whose entries bring ``counts`` tokens is cut: a list of pieces, each a list
+        of ``(entry, first token, one past the last token)`` in the order of the entries."""
+        pieces: List[List[tuple]] = []
+        done = [0] * len(counts)
+        while any(d < c for d, c in zip(done, counts)):
+            room = self.max_step_tokens
+            piece = []
+            for i, c in enumerate(counts):
+                left = c - done[i]
+                if left == 0 or room == 0:
+                    continue
+                take = min(left, room)
+                piece.append((i, done[i], done[i] + take))
+                done[i] += take
+                room -= take
+            pieces.append(piece)
+        return pieces
 
     def _run_piece(self, slots: List[int], starts: List[int], tokens: List[List[int]],
                    want: List[List[int]]) -> Optional[torch.Tensor]:

@@ -62,16 +62,17 @@ class EngineBackend:
         self.sampler = sampler or DeviceSampler(engine.model.device)
         self.max_positions = engine.model.spec.max_positions
 
-    def can_admit(self, lengths: Sequence[int]) -> bool:
-        """Whether sequences that will grow to ``lengths`` fit beside nothing else."""
+    def can_admit(self, lengths: Sequence[int], prompts: Optional[Sequence[int]] = None) -> bool:
+        """Whether new sequences with prompts of ``prompts`` tokens that will grow to ``lengths``
+        fit the free slots and pages: the prompt step as the engine would cut it, then a token
+        at a time (a group with a window is counted by its window, not by the final length)."""
         cache = self.engine.cache
         if len(lengths) > cache.slots.n_free:
             return False
-        from ..cache import pages_for
-        for g in cache.kv_groups:
-            if sum(pages_for(n, g.page_size) for n in lengths) > g.n_free_pages:
-                return False
-        return True
+        prompts = list(lengths) if prompts is None else list(prompts)
+        keys = [("new", i) for i in range(len(lengths))]
+        pieces = [[(keys[i], hi) for i, _, hi in piece] for piece in self.engine.plan_pieces(prompts)]
+        return cache.fits(pieces, final=list(zip(keys, lengths))) is None
 
     def new_sequence(self) -> int:
         return self.engine.new_sequence()
@@ -98,6 +99,7 @@ class _Live:
     slot: int
     sampling: SequenceSampling
     out: List[int] = field(default_factory=list)
+    released: bool = False
 
 
 class Generator:
@@ -107,6 +109,9 @@ class Generator:
         self.backend = backend
         self.max_batch = max_batch
         self.stats = GenerateStats()
+        # called with the number of decode steps run so far after each of them: a place for a
+        # benchmark to take its times without a loop of its own
+        self.on_step = None
 
     def _final_length(self, r: Request) -> int:
         return min(len(r.prompt) + r.max_new_tokens, self.backend.max_positions)
@@ -114,6 +119,7 @@ class Generator:
     def _take_batch(self, requests: Sequence[Request], first: int) -> int:
         """Number of requests, from ``first`` on, that start together."""
         lengths: List[int] = []
+        prompts: List[int] = []
         n = 0
         while first + n < len(requests) and n < self.max_batch:
             r = requests[first + n]
@@ -121,12 +127,10 @@ class Generator:
                 if n == 0:
                     return 0      # handled alone by the caller
                 break
-            if len(r.prompt) > self.backend.max_positions:
-                raise RocmlError(f"request {first + n}: a prompt of {len(r.prompt)} tokens exceeds the "
-                                 f"model's {self.backend.max_positions} positions")
-            if not self.backend.can_admit(lengths + [self._final_length(r)]):
+            if not self.backend.can_admit(lengths + [self._final_length(r)], prompts + [len(r.prompt)]):
                 break
             lengths.append(self._final_length(r))
+            prompts.append(len(r.prompt))
             n += 1
         if n == 0:
             raise CacheFullError(f"request {first} does not fit the cache even alone "
@@ -134,6 +138,12 @@ class Generator:
         return n
 
     def run(self, requests: Sequence[Request]) -> List[Result]:
+        # every request is looked at before the first batch starts: a request that can never run
+        # must not cost the results of those before it
+        for i, r in enumerate(requests):
+            if len(r.prompt) > self.backend.max_positions:
+                raise RocmlError(f"request {i}: a prompt of {len(r.prompt)} tokens exceeds the "
+                                 f"model's {self.backend.max_positions} positions")
         results: List[Optional[Result]] = [None] * len(requests)
         at = 0
         while at < len(requests):
@@ -150,9 +160,21 @@ class Generator:
 
     def _run_batch(self, requests, first: int, n: int, results) -> None:
         be = self.backend
-        live = [_Live(first + i, requests[first + i], be.new_sequence(),
-                      SequenceSampling.start(requests[first + i].params, first + i, requests[first + i].prompt))
-                for i in range(n)]
+        live: List[_Live] = []
+        try:
+            for i in range(n):
+                r = requests[first + i]
+                live.append(_Live(first + i, r, be.new_sequence(), SequenceSampling.start(r.params, first + i, r.prompt)))
+            self._decode_batch(live, results)
+        finally:
+            # whatever ended the batch, its sequences give their slots and pages back
+            for s in live:
+                if not s.released:
+                    s.released = True
+                    be.release(s.slot)
+
+    def _decode_batch(self, live: List[_Live], results) -> None:
+        be = self.backend
         self.stats.batches += 1
         t0 = time.perf_counter()
         logits = be.step([s.slot for s in live], [list(s.request.prompt) for s in live])
@@ -160,10 +182,11 @@ class Generator:
         t1 = time.perf_counter()
         self.stats.prompt_seconds += t1 - t0
         self.stats.prompt_tokens += sum(len(s.request.prompt) for s in live)
-        while live:
-            drawn = be.sample(logits, [s.sampling for s in live])
+        running = list(live)
+        while running:
+            drawn = be.sample(logits, [s.sampling for s in running])
             still: List[_Live] = []
-            for s, tok in zip(live, drawn):
+            for s, tok in zip(running, drawn):
                 reason = None
                 if s.request.max_new_tokens <= 0:
                     reason = "length"
@@ -181,10 +204,13 @@ class Generator:
                     still.append(s)
                 else:
                     results[s.index] = Result(s.out, reason, len(s.request.prompt))
+                    s.released = True
                     be.release(s.slot)
-            live = still
-            if live:
-                logits = be.step([s.slot for s in live], [[s.out[-1]] for s in live])
+            running = still
+            if running:
+                logits = be.step([s.slot for s in running], [[s.out[-1]] for s in running])
                 self.stats.decode_steps += 1
+                if self.on_step is not None:
+                    self.on_step(self.stats.decode_steps)
         be.synchronize()
         self.stats.decode_seconds += time.perf_counter() - t1

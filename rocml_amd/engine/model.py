@@ -11,10 +11,14 @@ import torch
 
 from .. import ops
 from ..cache import Cache, CacheLineView, KVGroup
+from ..cache.cache import HEADROOM_BYTES
 from ..config.spec import ModelSpec
 from ..errors import ConfigError
 from ..parts import BuildContext, ParamSpec, build_block, build_norm
 from .batch import StepContext
+from .workspace import Workspace
+
+RUNTIME_BYTES = 256 << 20      # kept free for the runtime, code objects and the sampler beside the activations
 
 _DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32,
            torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
@@ -80,13 +84,32 @@ class DecoderModel:
         return [None if e.reads_cache_of is not None else self.blocks[e.layer].cache_request()
                 for e in self.spec.schedule]
 
-    def new_cache(self, max_tokens: int, max_seqs: Optional[int] = None) -> Cache:
+    def activation_bytes(self, n_tokens: int, n_wanted: int) -> int:
+        """Bytes of activations and scratch memory a step of ``n_tokens`` tokens with ``n_wanted``
+        rows of logits asks the workspace for: the residual stream, the largest layer's buffers
+        (layers share theirs), the wanted rows and their logits, and the scratch memory."""
+        s = self.spec
+        size = torch.empty((), dtype=self.dtype).element_size()
+        per_layer = max(b.activation_bytes(n_tokens) for b in self.blocks)
+        return (n_tokens * s.hidden * 4 + per_layer + n_wanted * (s.hidden * size + s.vocab * 4)
+                + Workspace.SCRATCH_BYTES)
+
+    def new_cache(self, max_tokens: int, max_seqs: Optional[int] = None,
+                  step_tokens: Optional[int] = None) -> Cache:
+        """The cache for this model.  ``step_tokens`` (the most tokens a piece of a step brings)
+        sizes what is left free beside the cache: the reference's 768 MiB
+        (rocml/src/budget/mod.rs:37) cover its pieces of 512 tokens, a longer piece needs more."""
         free = None
         if torch.device(self.device).type == "cuda":
             # what the driver reports as free, and what torch holds without using it
             free = torch.cuda.mem_get_info(self.device)[0] + \
                 torch.cuda.memory_reserved(self.device) - torch.cuda.memory_allocated(self.device)
-        return Cache(self.cache_requests(), max_tokens, self.dtype, self.device, max_seqs=max_seqs, free_bytes=free)
+        headroom = HEADROOM_BYTES
+        if step_tokens is not None:
+            wanted = max_seqs if max_seqs is not None else 64
+            headroom = max(headroom, self.activation_bytes(step_tokens, wanted) + RUNTIME_BYTES)
+        return Cache(self.cache_requests(), max_tokens, self.dtype, self.device, max_seqs=max_seqs,
+                     free_bytes=free, step_tokens=step_tokens, headroom=headroom)
 
     # -- forward -----------------------------------------------------------------------
     def forward(self, step: StepContext, cache: Cache, block_tables: Dict[str, torch.Tensor],

@@ -17,7 +17,9 @@ import torch
 
 
 class Workspace:
-    def __init__(self, device, scratch_bytes: int = 128 << 20):
+    SCRATCH_BYTES = 128 << 20
+
+    def __init__(self, device, scratch_bytes: int = SCRATCH_BYTES):
         self.device = device
         self._buffers: Dict[str, torch.Tensor] = {}
         self.generation = 0

@@ -60,6 +60,11 @@ class Attention(Mixer):
             self.q_gain = tensors["q_norm.weight"]
             self.k_gain = tensors["k_norm.weight"]
 
+    def activation_bytes(self, n_tokens: int) -> int:
+        size = 2 if self.dtype == torch.bfloat16 else 4
+        rot = 0 if self.position is None else 2 * n_tokens * (self.position.rot_dim // 2) * 4
+        return n_tokens * ((self.q_dim + 2 * self.kv_dim) * 4 + 2 * self.q_dim * size) + rot
+
     def cache_request(self) -> KVCacheRequest:
         return KVCacheRequest(self.spec.n_kv_heads, self.spec.head_dim, self.spec.window)
 

@@ -69,6 +69,11 @@ class Part:
         """Receives the tensors named by ``param_specs``, already on the device and in
         the type their role asks for."""
 
+    def activation_bytes(self, n_tokens: int) -> int:
+        """Bytes of workspace buffers the part asks for in a step of ``n_tokens`` tokens; what
+        the cache leaves free beside itself is sized with it."""
+        return 0
+
 
 class Norm(Part):
     def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:

@@ -17,6 +17,7 @@ from .registry import build_feed_forward, build_mixer, build_norm, register_bloc
 class PreNormBlock(Part):
     def __init__(self, spec: BlockSpec, ctx: BuildContext):
         self.dtype = ctx.dtype
+        self.hidden = spec.mixer_norm.size
         self.children = {"mixer_norm": build_norm(spec.mixer_norm, ctx),
                          "mixer": build_mixer(spec.mixer, ctx),
                          "ffn_norm": build_norm(spec.ffn_norm, ctx),
@@ -37,6 +38,10 @@ class PreNormBlock(Part):
 
     def cache_request(self):
         return self.mixer.cache_request()
+
+    def activation_bytes(self, n_tokens: int) -> int:
+        size = 2 if self.dtype == torch.bfloat16 else 4
+        return n_tokens * self.hidden * size + self.mixer.activation_bytes(n_tokens) + self.ffn.activation_bytes(n_tokens)
 
     def forward(self, step, x: torch.Tensor, cache, owns_cache: bool) -> None:
         xn = step.workspace.get("block.xn", tuple(x.shape), self.dtype)

@@ -38,6 +38,12 @@ class GatedMlp(FeedForward):
         self.w_down = tensors["down_proj.weight"]
         self.fused = self.dtype == torch.bfloat16 and self.spec.hidden % 8 == 0
 
+    def activation_bytes(self, n_tokens: int) -> int:
+        s = self.spec
+        size = 2 if self.dtype == torch.bfloat16 else 4
+        fused = self.dtype == torch.bfloat16 and s.hidden % 8 == 0
+        return n_tokens * s.intermediate * (size + (0 if fused else 8))
+
     def forward(self, step, xn, x_accum) -> None:
         s = self.spec
         n = step.n_tokens

@@ -102,7 +102,8 @@ def load_model(path: str, dtype="bfloat16", device="cuda") -> DecoderModel:
 
 def random_model(config: Dict, seed: int, dtype="bfloat16", device="cuda", norm_jitter: bool = False,
                  n_layers: Optional[int] = None) -> DecoderModel:
-    """A model with random weights drawn on the device, without a file (benchmarks)."""
+    """A model with random weights drawn on the device, without a file; the values are the ones
+    ``write_model_dir`` writes for the same configuration and seed."""
     from .random_init import random_tensor
     if n_layers is not None:
         config = dict(config, num_hidden_layers=n_layers)

@@ -21,21 +21,77 @@ STD = 0.02
 
 def _tensor_seed(seed: int, name: str) -> int:
     digest = hashlib.sha256(f"{seed}:{name}".encode("utf-8")).digest()
-    return int.from_bytes(digest[:8], "little") & ((1 << 63) - 1)
+    return int.from_bytes(digest[:8], "little")
+
+
+# The draws are the same bits on the CPU and on the GPU: element i of a tensor is a function of
+# (seed, tensor name, i) made of operations that every device computes exactly.  A counter-based
+# generator (splitmix64: a 64-bit counter times the golden-ratio increment, then two rounds of
+# xor-shift and multiply, all in wrapping 64-bit integers) gives 32 bits per element; the upper
+# 16 pick a cell of the inverse normal distribution function, tabulated once on the CPU, the
+# lower 16 a place inside the cell, by one multiplication and one addition in 64-bit floating
+# point.  The distribution is the normal one with its density made piecewise constant on 65,536
+# cells of equal probability and its tails cut near 5 standard deviations.
+_CELLS = 1 << 16
+_CHUNK = 1 << 26
+_table_cache: Dict[str, torch.Tensor] = {}
+
+
+def _signed(v: int) -> int:
+    v &= (1 << 64) - 1
+    return v - (1 << 64) if v >= (1 << 63) else v
+
+
+def _lsr(x: torch.Tensor, n: int) -> torch.Tensor:
+    return (x >> n) & ((1 << (64 - n)) - 1)
+
+
+def _quantile_table(device) -> torch.Tensor:
+    key = str(device)
+    if key not in _table_cache:
+        edges = torch.arange(_CELLS + 1, dtype=torch.float64) / _CELLS
+        edges[0], edges[-1] = 1.0 / (_CELLS * 64), 1.0 - 1.0 / (_CELLS * 64)
+        _table_cache[key] = torch.special.ndtri(edges).to(device)
+    return _table_cache[key]
+
+
+def standard_normal(n: int, stream: int, device="cpu") -> torch.Tensor:
+    """``n`` draws of stream ``stream`` (any 64-bit integer) as 64-bit floats on ``device``."""
+    table = _quantile_table(device)
+    out = torch.empty(n, dtype=torch.float64, device=device)
+    for start in range(0, n, _CHUNK):
+        stop = min(n, start + _CHUNK)
+        z = torch.arange(start + 1, stop + 1, dtype=torch.int64, device=device)
+        z = z * _signed(0x9E3779B97F4A7C15) + _signed(stream)
+        z = (z ^ _lsr(z, 30)) * _signed(0xBF58476D1CE4E5B9)
+        z = (z ^ _lsr(z, 27)) * _signed(0x94D049BB133111EB)
+        z = z ^ _lsr(z, 31)
+        cell = _lsr(z, 48)
+        inside = (_lsr(z, 32) & (_CELLS - 1)).to(torch.float64)
+        inside = (inside + 0.5) * (1.0 / _CELLS)
+        low = table[cell]
+        width = table[cell + 1] - low
+        out[start:stop] = low + width * inside
+    return out
 
 
 def random_tensor(name: str, spec: ParamSpec, seed: int, dtype: torch.dtype, norm_jitter: bool,
                   device="cpu") -> torch.Tensor:
-    """The tensor called ``name`` for ``seed``: drawn in 32-bit on ``device``, then cast.
-    The CPU and the GPU draw different values for the same seed; files are written on the CPU."""
-    gen = torch.Generator(device=device)
-    gen.manual_seed(_tensor_seed(seed, name))
+    """The tensor called ``name`` for ``seed``: drawn on ``device``, the same values on any device,
+    rounded once to ``dtype``."""
+    n = 1
+    for d in spec.shape:
+        n *= d
+
+    def normal() -> torch.Tensor:
+        return (standard_normal(n, _tensor_seed(seed, name), device) * STD).to(torch.float32).view(spec.shape)
+
     if spec.init == "normal":
-        t = torch.empty(spec.shape, dtype=torch.float32, device=device).normal_(0.0, STD, generator=gen)
+        t = normal()
     elif spec.init == "gain":
         t = torch.ones(spec.shape, dtype=torch.float32, device=device)
         if norm_jitter:
-            t += torch.empty(spec.shape, dtype=torch.float32, device=device).normal_(0.0, STD, generator=gen)
+            t += normal()
     elif spec.init == "zeros":
         t = torch.zeros(spec.shape, dtype=torch.float32, device=device)
     else:

@@ -156,9 +156,14 @@ def test_storage_is_checked_against_free_memory_before_it_is_allocated():
     full = KVCacheRequest(n_kv_heads=8, head_dim=128, window=None)
     windowed = KVCacheRequest(n_kv_heads=2, head_dim=64, window=100)
     state = StateRequest(shape=(4, 16), dtype=torch.float32)
-    need = planned_bytes([full, full, None, windowed, state], max_tokens=64 * 1000, dtype=torch.bfloat16, max_seqs=10)
+    need = planned_bytes([full, full, None, windowed, state], max_tokens=64 * 1000, dtype=torch.bfloat16, max_seqs=10,
+                         step_tokens=640)
     kv_full = 2 * 2 * 64 * 1000 * 8 * 128 * 2                       # two lines of 1000 pages
-    kv_window = 2 * (10 * 3) * 64 * 2 * 64 * 2                      # a window of 100 is two pages and one more, per sequence
+    # a window of 100 is two pages, one more as it starts inside a page, one being filled, per
+    # sequence; and the ten pages of a piece's own 640 tokens
+    kv_window = 2 * (10 * 4 + 10) * 64 * 2 * 64 * 2
+    # without a bound on the pieces a windowed group is sized like one that keeps everything
+    assert planned_bytes([windowed], 64 * 1000, torch.bfloat16, max_seqs=10) == 2 * 1000 * 64 * 2 * 64 * 2
     assert need == kv_full + kv_window + 10 * 64 * 4
     check_budget(need, need + HEADROOM_BYTES)
     with pytest.raises(MemoryBudgetError, match="GiB free"):
@@ -167,3 +172,41 @@ def test_storage_is_checked_against_free_memory_before_it_is_allocated():
         Cache([full], max_tokens=1 << 40, dtype=torch.bfloat16, device="cpu", free_bytes=1 << 30)
     cache = Cache([full], max_tokens=128, dtype=torch.float32, device="cpu", free_bytes=HEADROOM_BYTES + (1 << 20))
     assert cache.n_pages == 2
+
+
+def test_a_windowed_group_takes_prompts_far_longer_than_its_window():
+    """Pieces are reserved and committed one after the other; the windowed group, sized for its
+    windows and one piece, gives pages back between them, and the plan is checked as a whole
+    before anything is reserved."""
+    full = KVCacheRequest(n_kv_heads=1, head_dim=16, window=None)
+    windowed = KVCacheRequest(n_kv_heads=1, head_dim=16, window=70)
+    c = Cache([full, windowed], max_tokens=4096, dtype=torch.float32, device="cpu", max_seqs=2, step_tokens=256)
+    g_full, g_win = c.kv_groups
+    assert g_full.n_pages == 64 and g_win.n_pages == 2 * 4 + 4
+    a, b = c.new_sequence(), c.new_sequence()
+    pieces = [[(a, 256)], [(a, 512)], [(a, 768)], [(a, 1000), (b, 24)], [(b, 280)], [(b, 300)]]
+    assert c.fits(pieces) is None
+    for piece in pieces:
+        slots, lens = [s for s, _ in piece], [n for _, n in piece]
+        c.reserve(slots, lens)
+        c.commit(slots, lens)
+        c.check()
+        for s, n in piece:                                         # the window's pages are all held
+            table = g_win.page_table(s)
+            assert all(p >= 0 for p in table[max(0, n - 70 + 1) // 64:])
+    assert c.length(a) == 1000 and c.length(b) == 300
+    assert g_win.n_pages - g_win.n_free_pages <= 2 * 3
+    # a token at a time to the end of the full group's room: never more than the window's pages
+    for n in range(1001, 1200):
+        c.reserve([a], [n])
+        c.commit([a], [n])
+    assert g_win.n_pages - g_win.n_free_pages <= 2 * 3
+    # a plan that does not fit is refused whole and says which group is short
+    short = c.fits([[(a, 1200 + 256)], [(a, 1200 + 512)], [(a, 4097)]])
+    assert short is not None and "kv0" in short
+    c.check()
+    # new sequences are counted from nothing; a final length counts a windowed group by its window
+    c.free_sequence(a)
+    c.free_sequence(b)
+    assert c.fits([[("x", 256)], [("x", 512)]], final=[("x", 4096)]) is None
+    assert c.fits([[("x", 256)]], final=[("x", 4097)]) is not None

@@ -21,7 +21,7 @@ class Scripted:
         self.step_tokens: List[List[List[int]]] = []
         self.released: List[int] = []
 
-    def can_admit(self, lengths):
+    def can_admit(self, lengths, prompts=None):
         return len(lengths) <= len(self.free_slots) and sum(lengths) <= self.room
 
     def new_sequence(self):
