@@ -5,10 +5,12 @@
 
 A step is one decode step of a batch of 8 sequences, each with a 2,048-token random
 prompt in the cache (context length 4,096): the engine's step over the cache, greedy
-sampling on the device and the copy of the drawn ids to the host, as generation does it.
+sampling on the device and the copy of the drawn ids to the host, exactly as the library's
+generation loop runs it (the loop is the one that is timed, through its per-step hook).
 Prints one JSON line: ``value`` is decoded tokens per second; ``prefill`` is one
 2,048-token prompt; ``roofline`` relates the decode step to the bytes it must read
-(every weight once and the live cache) at 8 TB/s; ``points`` holds batch 1 and 64.
+(every weight once and the live cache) at 8 TB/s; ``points`` holds batch 1 and 64 and
+``point_fracs`` their fractions of that roofline.
 The workload follows the reference's bench (rocml-cli/src/cmd_bench.rs:79-243): synthetic
 prompt, greedy, no stop token, warm-up first; times are taken around synchronised steps.
 """
@@ -46,25 +48,22 @@ def main() -> int:
     import torch
     from rocml_amd import ops
     from rocml_amd.config.catalog import resolve
-    from rocml_amd.engine import Engine, StepEntry
-    from rocml_amd.sampling import DeviceSampler, SamplingParams, SequenceSampling
+    from rocml_amd.engine import Engine, EngineBackend, Generator, Request, StepEntry
+    from rocml_amd.sampling import SamplingParams
     from rocml_amd.weights import random_model
 
     ops.load_all()
-    entry = resolve(args.model).entry
-    cfg_full = entry.config
-    model = random_model(cfg_full, seed=0, dtype=args.dtype, device="cuda:0", n_layers=args.layers)
-    cfg = model.config
+    raw = resolve(args.model).entry.config              # config.json's keys
+    model = random_model(raw, seed=0, dtype=args.dtype, device="cuda:0", n_layers=args.layers)
     spec = model.spec
-    n_layers = cfg.num_hidden_layers
+    n_layers = len(spec.schedule)
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
     max_batch = max(batches)
     engine = Engine(model, max_tokens=max_batch * CONTEXT, max_seqs=max_batch, max_step_tokens=8192)
-    sampler = DeviceSampler(model.device)
     rng = np.random.default_rng(0)
 
     def prompt():
-        return [int(t) for t in rng.integers(0, cfg.vocab_size, size=PROMPT_LEN)]
+        return [int(t) for t in rng.integers(0, spec.vocab, size=PROMPT_LEN)]
 
     def sync():
         torch.cuda.synchronize()
@@ -85,64 +84,67 @@ def main() -> int:
         prefill_once()
         times.append(time.perf_counter() - t0)
     prefill_s = sorted(times)[len(times) // 2]
-    lin = (cfg.q_dim + 2 * cfg.kv_dim) * cfg.hidden_size + cfg.hidden_size * cfg.q_dim \
-        + 3 * cfg.intermediate_size * cfg.hidden_size
-    prefill_flops = n_layers * (2 * PROMPT_LEN * lin
-                                + 4 * cfg.num_attention_heads * cfg.head_dim * PROMPT_LEN * (PROMPT_LEN + 1) // 2) \
-        + 2 * cfg.vocab_size * cfg.hidden_size
+    prefill_flops = model.step_flops([PROMPT_LEN], [0], 1)
     peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
 
     # ---- decode ----------------------------------------------------------------------
-    elem = 2 if args.dtype == "bfloat16" else 4
-    weight_bytes = (n_layers * lin + cfg.vocab_size * cfg.hidden_size) * elem
+    weight_bytes = model.step_weight_bytes()
     kv_bytes_per_token = engine.cache.bytes_per_token()
 
+    class SkippingBackend(EngineBackend):
+        """Hands the sequences their prompt's positions without running it."""
+
+        def step(self, slots, tokens):
+            if all(len(t) == 1 for t in tokens):
+                return super().step(slots, tokens)
+            for s, t in zip(slots, tokens):
+                self.engine.adopt_positions(s, len(t))
+            return torch.zeros((len(slots), spec.vocab), dtype=torch.float32, device=model.device)
+
     def decode(batch: int, steps: int, warmup: int):
-        slots = [engine.new_sequence() for _ in range(batch)]
-        greedy = [SequenceSampling.start(SamplingParams.greedy(), i, []) for i in range(batch)]
-        # All prompts in one step, as the generation loop sends them (the engine cuts the step
-        # into pieces of its own; the prefill is not what is timed here).
-        if args.skip_prompts:
-            engine.cache.reserve(slots, [PROMPT_LEN] * batch)
-            engine.cache.commit(slots, [PROMPT_LEN] * batch)
-            tokens = [1] * batch
-        else:
-            logits = engine.step([StepEntry(s, prompt(), [PROMPT_LEN - 1]) for s in slots])
-            tokens = sampler.sample(logits, greedy)
+        """Seconds of ``steps`` decode steps of the generation loop after ``warmup`` of them, and
+        the mean sequence length over the timed steps."""
+        backend = (SkippingBackend if args.skip_prompts else EngineBackend)(engine)
+        gen = Generator(backend, max_batch=batch)
+        marks = {}
 
-        def one_step(toks):
-            logits = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, toks)])
-            return sampler.sample(logits, greedy)
+        def on_step(k: int) -> None:
+            if k == warmup or k == warmup + steps:
+                sync()
+                marks[k] = time.perf_counter()
+        gen.on_step = on_step
+        greedy = SamplingParams.greedy()
+        # one token more than the steps: the last token of a sequence is drawn, not run
+        requests = [Request(prompt(), warmup + steps + 1, greedy) for _ in range(batch)]
+        results = gen.run(requests)
+        assert all(len(r.tokens) == warmup + steps + 1 for r in results) and gen.stats.batches == 1
+        mean_len = PROMPT_LEN + warmup + (steps + 1) / 2.0
+        return marks[warmup + steps] - marks[warmup], mean_len
 
-        for _ in range(warmup):
-            tokens = one_step(tokens)
-        sync()
-        len0 = engine.length(slots[0])
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            tokens = one_step(tokens)
-        sync()
-        dt = time.perf_counter() - t0
-        mean_len = len0 + (steps + 1) / 2.0
-        for s in slots:
-            engine.release(s)
-        return dt, mean_len
+    def roofline(batch: int, dt_step: float, mean_len: float):
+        step_bytes = weight_bytes + batch * mean_len * kv_bytes_per_token
+        return step_bytes / dt_step / 1e9
 
-    steps = max(1, min(args.steps, CONTEXT - PROMPT_LEN - args.warmup - 1))
+    steps = max(1, min(args.steps, CONTEXT - PROMPT_LEN - args.warmup - 2))
     dt, mean_len = decode(args.batch, steps, args.warmup)
     ms_per_step = dt / steps * 1e3
     value = args.batch * steps / dt
-    step_bytes = weight_bytes + args.batch * mean_len * kv_bytes_per_token
-    achieved = step_bytes / (dt / steps) / 1e9
-    points = {}
+    achieved = roofline(args.batch, dt / steps, mean_len)
+    points, fracs = {}, {}
     if not args.no_points:
         for b in (1, 64):
             if b == args.batch:
                 points[f"decode_b{b}"] = round(value, 2)
+                fracs[f"decode_b{b}"] = round(achieved / HBM_PEAK_GBS, 4)
                 continue
             p_steps = max(1, min(steps, 64))
-            p_dt, _ = decode(b, p_steps, min(args.warmup, 4))
+            p_warm = min(args.warmup, 4)
+            p_dt, p_len = decode(b, p_steps, p_warm)
             points[f"decode_b{b}"] = round(b * p_steps / p_dt, 2)
+            fracs[f"decode_b{b}"] = round(roofline(b, p_dt / p_steps, p_len) / HBM_PEAK_GBS, 4)
+
+    def key(name, default=None):
+        return raw.get(name, default)
 
     out = {
         "metric": f"decode tok/s ({args.model} shape, {'bf16' if args.dtype == 'bfloat16' else 'fp32'}, "
@@ -151,18 +153,19 @@ def main() -> int:
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: uniform random token ids, random N(0, 0.02) weights, unit norm gains",
-        "config": {"model": args.model, "layers": n_layers, "layers_of_model": cfg_full["num_hidden_layers"],
-                   "hidden": cfg.hidden_size, "q_heads": cfg.num_attention_heads,
-                   "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
-                   "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
-                   "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_norm_eps,
-                   "tied_lm_head": cfg.tie_word_embeddings, "global_batch": args.batch,
+        "config": {"model": args.model, "layers": n_layers, "layers_of_model": key("num_hidden_layers"),
+                   "hidden": spec.hidden, "q_heads": key("num_attention_heads"),
+                   "kv_heads": key("num_key_value_heads"), "head_dim": key("head_dim"),
+                   "intermediate": key("intermediate_size"), "vocab": spec.vocab,
+                   "rope_theta": key("rope_theta"), "rms_norm_eps": key("rms_norm_eps"),
+                   "tied_lm_head": spec.tie_lm_head, "global_batch": args.batch,
                    "prompt_len": PROMPT_LEN, "seq_len": CONTEXT, "parallelism": "single GPU"},
         "prefill": {"value": round(PROMPT_LEN / prefill_s, 1), "tokens": PROMPT_LEN,
                     "ms": round(prefill_s * 1e3, 3), "frac": round(prefill_flops / prefill_s / peak, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
         "points": points,
+        "point_fracs": fracs,
     }
     print(json.dumps(out))
     return 0

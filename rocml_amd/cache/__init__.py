@@ -1,3 +1,2 @@
-from .cache import Cache, CacheLineView, KVGroup, PAGE_SIZE, SlotAllocator, StateGroup, pages_for
-
-__all__ = ["Cache", "CacheLineView", "KVGroup", "PAGE_SIZE", "SlotAllocator", "StateGroup", "pages_for"]
+from .cache import (Cache, CacheGroup, CacheLineView, Geometry, KVGroup, PAGE_SIZE, PagedGroup, SlotAllocator,
+                    StateGroup, pages_for, register_cache_group)

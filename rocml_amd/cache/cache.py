@@ -74,24 +74,76 @@ class SlotAllocator:
         return frozenset(self._live)
 
 
-class KVGroup:
-    """Paged keys and values of the cache lines that share one ``KVCacheRequest``."""
+@dataclass(frozen=True)
+class Geometry:
+    """What a cache was asked to hold; every group sizes its storage from it."""
+    n_pages: int                  # pages of page_size positions for live sequences together
+    page_size: int
+    n_slots: int                  # most live sequences
+    max_seqs: Optional[int]       # the caller's bound on live sequences, if it gave one
+    step_tokens: Optional[int]    # most tokens one piece of a step brings, if bounded
+    dtype: torch.dtype            # the model's compute type
+    device: object
 
-    def __init__(self, name: str, request: KVCacheRequest, n_lines: int, n_pages: int,
-                 page_size: int, dtype: torch.dtype, device):
+
+class CacheGroup:
+    """Storage shared by the cache lines with one request.  The cache tells every group when a
+    sequence starts (``open``), reaches a length (``committed``) and ends (``close``); a group
+    hands a mixer its part of the storage with ``view``.  A group with ``paged`` true also keeps
+    a page table per sequence (``PagedGroup``)."""
+    paged = False
+
+    def __init__(self, name: str, request, n_lines: int):
         self.name = name
         self.request = request
         self.n_lines = n_lines
+
+    @staticmethod
+    def planned_bytes(request, n_lines: int, geo: "Geometry") -> int:
+        return 0
+
+    def open(self, slot: int) -> None:
+        pass
+
+    def committed(self, slot: int, length: int) -> None:
+        pass
+
+    def close(self, slot: int) -> None:
+        pass
+
+    def check(self) -> None:
+        pass
+
+    def view(self, line: int, step) -> "CacheLineView":
+        raise NotImplementedError
+
+
+class PagedGroup(CacheGroup):
+    """Page bookkeeping of a group that stores something per position: a pool of pages and, per
+    sequence, the pool pages of its logical pages.  ``window`` (None: everything is kept) lets
+    the group give pages back once no later query can see them.  Storage is the subclass's."""
+    paged = True
+
+    def __init__(self, name: str, request, n_lines: int, n_pages: int, page_size: int, window: Optional[int]):
+        super().__init__(name, request, n_lines)
         self.n_pages = n_pages
         self.page_size = page_size
-        # Values are transposed inside a page, which is the order the attention kernels
-        # multiply them in.  Zeroed once: rows beyond a sequence's length are never counted,
-        # but they are multiplied by a zero weight and so must stay finite.
-        h, d = request.n_kv_heads, request.head_dim
-        self.k = torch.zeros((n_lines, n_pages, h, page_size, d), dtype=dtype, device=device)
-        self.v = torch.zeros((n_lines, n_pages, h, d, page_size), dtype=dtype, device=device)
+        self.window = window
         self._free = list(range(n_pages - 1, -1, -1))
         self._pages: Dict[int, List[int]] = {}   # slot -> logical page -> pool page, -1 once released
+
+    @staticmethod
+    def pool_pages(window: Optional[int], geo: Geometry) -> int:
+        """Pages of the pool.  A group with a window holds, per sequence, the pages its window
+        spans (one more than the window's pages, as it rarely starts on a page's edge) and the
+        page being filled; while a step runs it also holds the pages of the step's own tokens,
+        which are only given back when the step's piece is committed.  With a bound on the
+        sequences and on the tokens of a piece the group needs no more than that, however long
+        the sequences grow; without them it is sized like a group that keeps everything."""
+        if window is not None and geo.max_seqs is not None and geo.step_tokens is not None:
+            return min(geo.n_pages, geo.max_seqs * (pages_for(window, geo.page_size) + 2)
+                       + pages_for(geo.step_tokens, geo.page_size))
+        return geo.n_pages
 
     # -- bookkeeping -----------------------------------------------------------------
     @property
@@ -125,10 +177,13 @@ class KVGroup:
                 if level < k:
                     self._pages[s].append(self._free.pop())
 
+    def committed(self, slot: int, length: int) -> None:
+        self.trim(slot, length)
+
     def trim(self, slot: int, length: int) -> None:
         """After a sequence reached ``length``: a group with a window releases the pages
         whose positions no query at ``length`` or later can see."""
-        w = self.request.window
+        w = self.window
         if w is None:
             return
         first_needed = max(0, length - w + 1) // self.page_size
@@ -155,21 +210,77 @@ class KVGroup:
                              f"({len(held)} held, {len(self._free)} free, {self.n_pages} in all)")
 
     def bytes_per_token(self) -> int:
+        return 0
+
+
+class KVGroup(PagedGroup):
+    """Paged keys and values of the cache lines that share one ``KVCacheRequest``."""
+
+    def __init__(self, name: str, request: KVCacheRequest, n_lines: int, geo: Geometry):
+        super().__init__(name, request, n_lines, self.pool_pages(request.window, geo), geo.page_size, request.window)
+        # Values are transposed inside a page, which is the order the attention kernels
+        # multiply them in.  Zeroed once: rows beyond a sequence's length are never counted,
+        # but they are multiplied by a zero weight and so must stay finite.
+        h, d = request.n_kv_heads, request.head_dim
+        self.k = torch.zeros((n_lines, self.n_pages, h, self.page_size, d), dtype=geo.dtype, device=geo.device)
+        self.v = torch.zeros((n_lines, self.n_pages, h, d, self.page_size), dtype=geo.dtype, device=geo.device)
+
+    @staticmethod
+    def planned_bytes(request: KVCacheRequest, n_lines: int, geo: Geometry) -> int:
+        size = torch.empty((), dtype=geo.dtype).element_size()
+        return (2 * n_lines * PagedGroup.pool_pages(request.window, geo) * geo.page_size
+                * request.n_kv_heads * request.head_dim * size)
+
+    def view(self, line: int, step) -> "CacheLineView":
+        return CacheLineView(group=self, line=line, k=self.k[line], v=self.v[line],
+                             block_table=step.block_tables[self.name])
+
+    def bytes_per_token(self) -> int:
         r = self.request
         return 2 * self.n_lines * r.n_kv_heads * r.head_dim * self.k.element_size()
 
 
-class StateGroup:
+class StateGroup(CacheGroup):
     """Fixed-size per-sequence state of the cache lines that share one ``StateRequest``."""
 
-    def __init__(self, name: str, request: StateRequest, n_lines: int, n_slots: int, device):
-        self.name = name
-        self.request = request
-        self.n_lines = n_lines
-        self.state = torch.zeros((n_lines, n_slots) + tuple(request.shape), dtype=request.dtype, device=device)
+    def __init__(self, name: str, request: StateRequest, n_lines: int, geo: Geometry):
+        super().__init__(name, request, n_lines)
+        self.state = torch.zeros((n_lines, geo.n_slots) + tuple(request.shape), dtype=request.dtype, device=geo.device)
+
+    @staticmethod
+    def planned_bytes(request: StateRequest, n_lines: int, geo: Geometry) -> int:
+        n = 1
+        for dim in request.shape:
+            n *= dim
+        return n_lines * geo.n_slots * n * torch.empty((), dtype=request.dtype).element_size()
 
     def open(self, slot: int) -> None:
         self.state[:, slot].zero_()
+
+    def view(self, line: int, step) -> "CacheLineView":
+        return CacheLineView(group=self, line=line, state=self.state[line], slots=step.seq_slots)
+
+
+# Which group class serves which kind of request.  A mixer with needs of its own brings a request
+# class and a group class (both may live outside this package) and registers the pair.
+_GROUP_KINDS: Dict[type, type] = {}
+
+
+def register_cache_group(request_type: type, group_type: type) -> None:
+    """``group_type(name, request, n_lines, geometry)`` builds the storage for ``request_type``;
+    its static ``planned_bytes(request, n_lines, geometry)`` says how much that will be."""
+    _GROUP_KINDS[request_type] = group_type
+
+
+def _group_type(req) -> type:
+    for rt, gt in _GROUP_KINDS.items():
+        if isinstance(req, rt):
+            return gt
+    raise RocmlError(f"unknown cache request {req!r}")
+
+
+register_cache_group(KVCacheRequest, KVGroup)
+register_cache_group(StateRequest, StateGroup)
 
 
 @dataclass
@@ -190,17 +301,19 @@ class CacheLineView:
 HEADROOM_BYTES = 768 << 20
 
 
-def _group_pages(req: KVCacheRequest, n_pages: int, max_seqs: Optional[int], page_size: int,
-                 step_tokens: Optional[int] = None) -> int:
-    """Pages of a key/value group.  A group with a window holds, per sequence, the pages its
-    window spans (one more than the window's pages, as it rarely starts on a page's edge) and
-    the page being filled; while a step runs it also holds the pages of the step's own tokens,
-    which are only given back when the step's piece is committed.  With a bound on the
-    sequences and on the tokens of a piece the group needs no more than that, however long
-    the sequences grow; without them it is sized like a group that keeps everything."""
-    if req.window is not None and max_seqs is not None and step_tokens is not None:
-        return min(n_pages, max_seqs * (pages_for(req.window, page_size) + 2) + pages_for(step_tokens, page_size))
-    return n_pages
+def _geometry(max_tokens: int, dtype, device, max_seqs: Optional[int], page_size: int,
+              step_tokens: Optional[int]) -> Geometry:
+    n_pages = max(1, pages_for(max_tokens, page_size))
+    return Geometry(n_pages=n_pages, page_size=page_size, n_slots=max_seqs if max_seqs is not None else n_pages,
+                    max_seqs=max_seqs, step_tokens=step_tokens, dtype=dtype, device=device)
+
+
+def _by_request(requests: Sequence[Optional[object]]) -> Dict[object, List[int]]:
+    by_request: Dict[object, List[int]] = {}
+    for entry, req in enumerate(requests):
+        if req is not None:
+            by_request.setdefault(req, []).append(entry)
+    return by_request
 
 
 def planned_bytes(requests: Sequence[Optional[object]], max_tokens: int, dtype: torch.dtype,
@@ -209,19 +322,9 @@ def planned_bytes(requests: Sequence[Optional[object]], max_tokens: int, dtype: 
     """Bytes the cache for these requests will allocate: per key/value line
     ``2 * pages * page_size * Hkv * D * bytes`` (rocml/src/budget/mod.rs:47-59), per state
     line ``slots * elements * bytes``."""
-    n_pages = max(1, pages_for(max_tokens, page_size))
-    slots = max_seqs if max_seqs is not None else n_pages
-    size = torch.empty((), dtype=dtype).element_size()
-    total = 0
-    for req in requests:
-        if isinstance(req, KVCacheRequest):
-            total += 2 * _group_pages(req, n_pages, max_seqs, page_size, step_tokens) * page_size * req.n_kv_heads * req.head_dim * size
-        elif isinstance(req, StateRequest):
-            n = 1
-            for dim in req.shape:
-                n *= dim
-            total += slots * n * torch.empty((), dtype=req.dtype).element_size()
-    return total
+    geo = _geometry(max_tokens, dtype, None, max_seqs, page_size, step_tokens)
+    return sum(_group_type(req).planned_bytes(req, len(entries), geo)
+               for req, entries in _by_request(requests).items())
 
 
 def check_budget(need: int, free: int, headroom: int = HEADROOM_BYTES, max_tokens: Optional[int] = None) -> None:
@@ -254,46 +357,39 @@ class Cache:
         if free_bytes is not None:
             check_budget(planned_bytes(requests, max_tokens, dtype, max_seqs, page_size, step_tokens), free_bytes,
                          headroom=headroom, max_tokens=max_tokens)
+        geo = _geometry(max_tokens, dtype, device, max_seqs, page_size, step_tokens)
         self.page_size = page_size
-        self.n_pages = max(1, pages_for(max_tokens, page_size))
-        self.max_seqs = max_seqs if max_seqs is not None else self.n_pages
+        self.n_pages = geo.n_pages
+        self.max_seqs = geo.n_slots
         self.slots = SlotAllocator(self.max_seqs)
         self.lengths: Dict[int, int] = {}
-        self.kv_groups: List[KVGroup] = []
-        self.state_groups: List[StateGroup] = []
-        self._line_of: Dict[int, Tuple[object, int]] = {}
-        by_request: Dict[object, List[int]] = {}
-        for entry, req in enumerate(requests):
-            if req is not None:
-                by_request.setdefault(req, []).append(entry)
-        for req, entries in by_request.items():
-            if isinstance(req, KVCacheRequest):
-                n_pages = _group_pages(req, self.n_pages, max_seqs, page_size, step_tokens)
-                name = f"kv{len(self.kv_groups)}" + ("" if req.window is None else f"w{req.window}")
-                group = KVGroup(name, req, len(entries), n_pages, page_size, dtype, device)
-                self.kv_groups.append(group)
-            elif isinstance(req, StateRequest):
-                group = StateGroup(f"state{len(self.state_groups)}", req, len(entries), self.max_seqs, device)
-                self.state_groups.append(group)
-            else:
-                raise RocmlError(f"unknown cache request {req!r}")
+        self.groups: List[CacheGroup] = []
+        self._line_of: Dict[int, Tuple[CacheGroup, int]] = {}
+        for req, entries in _by_request(requests).items():
+            kind = _group_type(req)
+            tag = kind.__name__.replace("Group", "").lower()
+            name = f"{tag}{sum(1 for g in self.groups if type(g) is kind)}"
+            if getattr(req, "window", None) is not None:
+                name += f"w{req.window}"
+            group = kind(name, req, len(entries), geo)
+            self.groups.append(group)
             for line, entry in enumerate(entries):
                 self._line_of[entry] = (group, line)
+        self.kv_groups: List[PagedGroup] = [g for g in self.groups if g.paged]       # every group with pages
+        self.state_groups: List[CacheGroup] = [g for g in self.groups if not g.paged]
 
     # -- sequences -------------------------------------------------------------------
     def new_sequence(self) -> int:
         slot = self.slots.alloc()
         self.lengths[slot] = 0
-        for g in self.kv_groups:
-            g.open(slot)
-        for g in self.state_groups:
+        for g in self.groups:
             g.open(slot)
         return slot
 
     def free_sequence(self, slot: int) -> None:
         self.slots.free(slot)
         del self.lengths[slot]
-        for g in self.kv_groups:
+        for g in self.groups:
             g.close(slot)
 
     def length(self, slot: int) -> int:
@@ -321,7 +417,7 @@ class Cache:
             free = g.n_free_pages
             size: Dict[object, int] = {}
             released: Dict[object, int] = {}
-            w = g.request.window
+            w = g.window
             for piece in pieces:
                 need = 0
                 for key, n in piece:
@@ -361,11 +457,11 @@ class Cache:
     def commit(self, slots: Sequence[int], new_lens: Sequence[int]) -> None:
         for s, n in zip(slots, new_lens):
             self.lengths[s] = n
-            for g in self.kv_groups:
-                g.trim(s, n)
+            for g in self.groups:
+                g.committed(s, n)
 
     # -- per step --------------------------------------------------------------------
-    def block_table(self, group: KVGroup, slots: Sequence[int], width: int) -> np.ndarray:
+    def block_table(self, group: PagedGroup, slots: Sequence[int], width: int) -> np.ndarray:
         table = np.full((len(slots), width), -1, dtype=np.int32)
         for row, slot in enumerate(slots):
             pages = group.page_table(slot)
@@ -382,8 +478,9 @@ class Cache:
         return entry in self._line_of
 
     def check(self) -> None:
-        for g in self.kv_groups:
+        for g in self.groups:
             g.check()
+        for g in self.kv_groups:
             if set(g._pages) != set(self.lengths):
                 raise RocmlError(f"cache group {g.name}: slots and page tables disagree")
         if set(self.lengths) != set(self.slots.live):

@@ -108,34 +108,45 @@ def cmd_bench(args) -> int:
     (rocml-cli/src/cmd_bench.rs:79-243)."""
     import numpy as np
     prompt_tokens = args.depth if args.depth is not None else args.prompt_tokens
+    if args.prompt_range is not None:
+        if not 1 <= args.prompt_range[0] <= args.prompt_range[1]:
+            raise RocmlError("--prompt-range needs 1 <= LO <= HI")
+        prompt_tokens = args.prompt_range[1]
     ctx = args.ctx or max(4096, prompt_tokens + args.decode_tokens)
     model = _load(args, ctx)
-    rng = np.random.default_rng(0)
+    rng = np.random.default_rng(args.prompt_seed)
     prefill, decode = [], []
     # Only the last run is profiled; it still counts for the medians, as in the reference
     # (rocml-cli/src/cmd_bench.rs:129-141), though its steps run launch by launch.
     want_profile = args.profile or args.profile_json is not None
     report = None
     for run in range(args.runs):
-        prompts = [[int(t) for t in rng.integers(0, model.vocab_size, size=prompt_tokens)]
-                   for _ in range(args.batch)]
+        if args.prompt_range is not None:
+            # unequal prompts, lengths uniform in [LO, HI], the same in every run of a seed
+            lo, hi = args.prompt_range
+            lengths = [int(n) for n in rng.integers(lo, hi + 1, size=args.batch)]
+        else:
+            lengths = [prompt_tokens] * args.batch
+        prompts = [[int(t) for t in rng.integers(0, model.vocab_size, size=n)] for n in lengths]
         if want_profile and run + 1 == args.runs:
             with _profiler(args.dtype) as profiler:
-                model.generate(prompts, max_new_tokens=args.decode_tokens)
+                model.generate(prompts, max_new_tokens=args.decode_tokens, ignore_eos=True)
             report = profiler.finish()
         else:
-            model.generate(prompts, max_new_tokens=args.decode_tokens)
+            model.generate(prompts, max_new_tokens=args.decode_tokens, ignore_eos=True)
         s = model.last_stats
         prefill.append(s.prompt_tok_s())
         decode.append(s.decode_tok_s())
-    out = {"model": args.model, "dtype": args.dtype, "batch": args.batch, "prompt_tokens": prompt_tokens,
+    out = {"model": args.model, "dtype": args.dtype, "batch": args.batch,
+           "prompt_tokens": prompt_tokens if args.prompt_range is None else sorted(lengths),
            "decode_tokens": args.decode_tokens, "runs": args.runs,
            "prefill_tok_s": statistics.median(prefill), "decode_tok_s": statistics.median(decode)}
     if args.json:
         print(json.dumps(out))
     else:
+        shown = f"{prompt_tokens} tokens" if args.prompt_range is None else f"{min(lengths)} to {max(lengths)} tokens"
         print(f"{args.model} {args.dtype} batch {args.batch}: prefill {out['prefill_tok_s']:.1f} tok/s "
-              f"({prompt_tokens} tokens), decode {out['decode_tok_s']:.1f} tok/s ({args.decode_tokens} tokens), "
+              f"({shown}), decode {out['decode_tok_s']:.1f} tok/s ({args.decode_tokens} tokens), "
               f"median of {args.runs}")
     if report is not None and args.profile:
         print(report.to_human())
@@ -145,17 +156,32 @@ def cmd_bench(args) -> int:
     return 0
 
 
+def _describe(spec) -> str:
+    """A part's spec in a few words: its kind and its sizes (the width it shares with the model
+    left out)."""
+    import dataclasses
+    if not dataclasses.is_dataclass(spec):
+        return getattr(spec, "kind", type(spec).__name__)
+    fields = [f"{f.name}={getattr(spec, f.name)}" for f in dataclasses.fields(spec)
+              if f.name not in ("kind", "hidden") and isinstance(getattr(spec, f.name), (int, str)) and not isinstance(getattr(spec, f.name), bool)]
+    return f"{spec.kind}({', '.join(fields)})"
+
+
 def cmd_models(args) -> int:
-    """Lists the catalog (rocml-cli/src/cmd_models.rs:13-38 prints name, family, presence)."""
-    from ..config import Qwen3Config
+    """Lists the catalog (rocml-cli/src/cmd_models.rs:13-38 prints name, family, presence); every
+    figure comes from the model that the entry's architecture builds, without weights."""
+    import torch
+    from ..config import architecture_of
     from ..config.catalog import CATALOG
-    print(f"{'name':<12} {'architecture':<18} {'layers':>6} {'hidden':>6} {'heads':>7} {'head':>5} "
-          f"{'inter':>6} {'vocab':>7} {'params':>9} {'bf16 GB':>8}")
+    from ..engine.model import DecoderModel
+    print(f"{'name':<12} {'architecture':<18} {'layers':>6} {'hidden':>6} {'vocab':>7} {'params':>9} {'bf16 GB':>8}  first layer")
     for e in CATALOG:
-        c = Qwen3Config.from_dict(e.config)
-        print(f"{e.name:<12} {c.architectures[0]:<18} {c.num_hidden_layers:>6} {c.hidden_size:>6} "
-              f"{c.num_attention_heads:>3}/{c.num_key_value_heads:<3} {c.head_dim:>5} {c.intermediate_size:>6} "
-              f"{c.vocab_size:>7} {c.n_params() / 1e9:>8.3f}B {c.n_params() * 2 / 1e9:>8.2f}")
+        arch = architecture_of(e.config)
+        spec = arch.to_spec(arch.read_config(e.config))
+        model = DecoderModel(spec, torch.bfloat16, device="meta")
+        first = spec.layers[spec.schedule[0].layer]
+        print(f"{e.name:<12} {spec.architecture:<18} {len(spec.schedule):>6} {spec.hidden:>6} {spec.vocab:>7} "
+              f"{model.n_params() / 1e9:>8.3f}B {model.weight_bytes() / 1e9:>8.2f}  {_describe(first.mixer)}, {_describe(first.ffn)}")
     return 0
 
 
@@ -170,7 +196,7 @@ def cmd_init(args) -> int:
     config = found.entry.config if found.entry is not None else read_config_json(found.path)
     jitter = found.entry.init_norm_jitter if found.entry is not None else True
     dtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
-    path = write_model_dir(args.out, config, args.weights_seed, dtype=dtype, norm_jitter=jitter)
+    path = write_model_dir(args.out, config, args.weights_seed, dtype=dtype, norm_jitter=jitter, device=args.device)
     print(path)
     return 0
 
@@ -199,6 +225,10 @@ def build_parser() -> argparse.ArgumentParser:
     b.add_argument("--runs", type=int, default=3)
     b.add_argument("--depth", type=int, default=None, help="prompt of this many tokens, then decode")
     b.add_argument("--ctx", type=int, default=None)
+    b.add_argument("--prompt-range", type=int, nargs=2, default=None, metavar=("LO", "HI"),
+                   help="unequal prompts: every sequence's length drawn uniformly from LO..HI")
+    b.add_argument("--prompt-seed", type=int, default=0, help="seed of the synthetic prompts")
+    b.add_argument("--weights-seed", type=int, default=0, help="seed of the random weights of a catalog model")
     b.add_argument("--json", action="store_true")
     b.add_argument("--profile", action="store_true", help="time every operation of the last run and print a roofline report")
     b.add_argument("--profile-json", default=None, metavar="PATH", help="write that report as JSON (implies profiling)")
@@ -210,6 +240,7 @@ def build_parser() -> argparse.ArgumentParser:
     i.add_argument("--out", required=True, help="folder to write config.json and model.safetensors to")
     i.add_argument("--weights-seed", type=int, default=0)
     i.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"], help="storage type of the tensors")
+    i.add_argument("--device", default="cpu", help="where the values are drawn (the same on any device); cuda:0 is faster for large models")
     i.set_defaults(fn=cmd_init)
     return ap
 

@@ -16,7 +16,6 @@ from typing import Dict, List, Optional
 
 from ..errors import UnknownModelError
 from ..sampling.params import SamplingParams
-from .qwen3 import ARCHITECTURE
 
 # Sampling preset the reference attaches to every dense Qwen3 entry
 # (rocml/src/registry/catalog.rs:44-51).
@@ -35,7 +34,7 @@ class ModelEntry:
 
 
 def _qwen3(vocab, hidden, inter, layers, heads, kv_heads, head_dim, theta, eps, tied, max_pos):
-    return {"architectures": [ARCHITECTURE], "model_type": "qwen3", "vocab_size": vocab,
+    return {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "vocab_size": vocab,
             "hidden_size": hidden, "intermediate_size": inter, "num_hidden_layers": layers,
             "num_attention_heads": heads, "num_key_value_heads": kv_heads, "head_dim": head_dim,
             "rope_theta": theta, "rms_norm_eps": eps, "tie_word_embeddings": tied,
@@ -58,7 +57,17 @@ CATALOG: List[ModelEntry] = [
 _BY_NAME = {e.name: e for e in CATALOG}
 
 
+def register_model(entry: ModelEntry) -> None:
+    """Adds a named configuration (of any registered architecture) to the catalog."""
+    if entry.name in _BY_NAME:
+        raise ValueError(f"the catalog already has a model called {entry.name!r}")
+    CATALOG.append(entry)
+    _BY_NAME[entry.name] = entry
+
+
 def catalog_names() -> List[str]:
+    from .registry import load_plugins
+    load_plugins()
     return [e.name for e in CATALOG]
 
 
@@ -76,6 +85,8 @@ class Resolved:
 
 
 def resolve(name_or_path: str) -> Resolved:
+    from .registry import load_plugins
+    load_plugins()
     if looks_like_path(name_or_path):
         if not os.path.isfile(os.path.join(name_or_path, "config.json")):
             raise UnknownModelError(f"{name_or_path!r} is not a model folder (no config.json in it)")

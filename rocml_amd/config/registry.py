@@ -30,6 +30,29 @@ class Architecture:
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
+_plugins_loaded = False
+
+PLUGINS_ENV = "ROCML_AMD_PLUGINS"
+
+
+def load_plugins() -> None:
+    """Imports the modules named in the environment variable ``ROCML_AMD_PLUGINS`` (separated by
+    commas), once.  A module that brings another architecture, parts or catalog entries registers
+    them when it is imported; this is how the command line and the replay program, which build
+    their model from config.json alone, learn of it without a change to this package."""
+    global _plugins_loaded
+    if _plugins_loaded:
+        return
+    _plugins_loaded = True
+    import importlib
+    for name in os.environ.get(PLUGINS_ENV, "").split(","):
+        name = name.strip()
+        if not name:
+            continue
+        try:
+            importlib.import_module(name)
+        except ImportError as e:
+            raise ConfigError(f"{PLUGINS_ENV} names the module {name!r}, which cannot be imported: {e}") from e
 
 
 def register_architecture(arch: Architecture) -> None:
@@ -37,10 +60,12 @@ def register_architecture(arch: Architecture) -> None:
 
 
 def known_architectures():
+    load_plugins()
     return sorted(_ARCHITECTURES)
 
 
 def architecture(name: str) -> Architecture:
+    load_plugins()
     if name not in _ARCHITECTURES:
         raise UnsupportedArchitectureError(
             f"architecture {name!r} is not registered; known: {', '.join(known_architectures())}")

@@ -107,14 +107,15 @@ static bool mfma_head_dim(int d) { return d == 32 || d == 64 || d == 96 || d == 
 
 // algo: 0 = choose, 1 = plain kernel, 2 = MFMA kernels (error if they cannot take the shapes).
 // cu_seqlens [n_seqs + 1] gives where each sequence's query tokens start (tokens of a sequence
-// are consecutive and in position order); max_new is the most query tokens of any sequence,
-// total_q_tiles the sum over sequences of ceil(tokens / 128), max_len the longest context.
+// are consecutive and in position order) and q_counts, an array in host memory, how many each has
+// (the prefill kernel's grid is sized from it); max_new is the most query tokens of any
+// sequence, max_len the longest context.
 // workspace holds the partial results of split decode attention.
 ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, const void* vcache,
                                  int dtype, const int* block_table, int bt_width,
                                  const int* token_seq, const int* token_pos, int n_tokens, int hq,
                                  int hkv, int d, int page_size, float scale, int window, int algo,
-                                 const int* cu_seqlens, int n_seqs, int max_new, int total_q_tiles,
+                                 const int* cu_seqlens, int n_seqs, int max_new, const int* q_counts,
                                  int max_len, int n_splits, void* workspace, long long workspace_bytes,
                                  hipStream_t stream) {
     ROCML_REQUIRE(n_tokens >= 0 && hq > 0 && hkv > 0 && d > 0 && page_size > 0 && bt_width > 0,
@@ -127,6 +128,16 @@ ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, c
     ROCML_REQUIRE(algo >= ATTN_AUTO && algo <= ATTN_MFMA, "attention: unknown algorithm %d", algo);
     if (n_tokens == 0) return 0;
     bool decode = max_new == 1;
+    long long total_q_tiles = 0, counted = 0;
+    if (q_counts && n_seqs > 0)
+        for (int b = 0; b < n_seqs; ++b) {
+            ROCML_REQUIRE(q_counts[b] >= 0, "attention: sequence %d has %d query tokens", b, q_counts[b]);
+            total_q_tiles += (q_counts[b] + AM_QTILE - 1) / AM_QTILE;
+            counted += q_counts[b];
+        }
+    ROCML_REQUIRE(!q_counts || n_seqs <= 0 || counted == n_tokens,
+                  "attention: the sequences' query counts add up to %lld, the step has %d tokens", counted, n_tokens);
+    ROCML_REQUIRE(total_q_tiles * hq < (1ll << 31), "attention: too many query tiles");
     bool mfma_ok = dtype == ROCML_BF16 && page_size == AM_PAGE && mfma_head_dim(d) && max_new >= 1 &&
                    (decode ? hq / hkv <= 16 : (cu_seqlens != nullptr && n_seqs > 0 && total_q_tiles > 0));
     if (algo == ATTN_MFMA)
@@ -135,7 +146,7 @@ ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, c
                                "the sequence offsets in prefill (D=%d page=%d group=%d)", d, page_size, hq / hkv);
     if (mfma_ok && algo != ATTN_PLAIN) {
         AttnArgs a{(const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table,
-                   bt_width, token_seq, token_pos, cu_seqlens, n_seqs, n_tokens, total_q_tiles, max_len, hq, hkv,
+                   bt_width, token_seq, token_pos, cu_seqlens, n_seqs, n_tokens, (int)total_q_tiles, max_len, hq, hkv,
                    scale, window, workspace, workspace_bytes, n_splits, nullptr};
         int rc = decode ? BY_HEAD_DIM(launch_decode_plain, d, a, stream) : BY_HEAD_DIM(launch_prefill, d, a, stream);
         if (rc) return rc;

@@ -395,9 +395,10 @@ __global__ void attn_decode_reduce_kernel(const float* __restrict__ part_o, cons
 }
 
 // ---- prefill: many query tokens per sequence --------------------------------------------------
-// grid: query tiles of 128 rows over all sequences x Hq, 4 waves of 32 query rows.  Pages of
+// grid: query tiles of AM_QTILE rows over all sequences x Hq, 4 waves of 32 query rows.  Pages of
 // keys and values go through LDS once per block; every wave multiplies its 32 queries with them.
 constexpr int AM_ROUND = 256;                           // blocks that start together: one per CU
+constexpr int AM_QTILE = 128;                           // query rows of a block: 32 per wave
 
 template <int D>
 struct PrefillLds {
@@ -437,14 +438,14 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     for (; b < n_seqs; ++b) {
         tok0 = cu_seqlens[b];
         n_new = cu_seqlens[b + 1] - tok0;
-        int tiles = (n_new + 127) / 128;
+        int tiles = (n_new + AM_QTILE - 1) / AM_QTILE;
         if (tile < tiles) break;
         tile -= tiles;
     }
     if (b >= n_seqs) return;
     const int* pages = block_table + (size_t)b * bt_width;
     int pos0 = token_pos[tok0];                        // position of the sequence's first new token
-    int row_lo = tile * 128, row_hi = min(n_new, row_lo + 128) - 1;     // block's query rows
+    int row_lo = tile * AM_QTILE, row_hi = min(n_new, row_lo + AM_QTILE) - 1;     // block's query rows
     int w_lo = row_lo + wave * 32, w_hi = min(n_new - 1, w_lo + 31);    // wave's query rows
     bool wave_active = w_lo < n_new;
     int my_row = w_lo + col;

@@ -37,7 +37,7 @@ class StepContext:
     seq_slots: torch.Tensor      # [B] int32: cache slot of each sequence
     max_new: int                 # most new tokens of any sequence
     max_len: int                 # longest sequence after this step
-    total_q_tiles: int           # sum over sequences of ceil(new tokens / 128)
+    new_counts: Sequence[int]    # new tokens of each sequence (host)
     workspace: Workspace
     memo: Dict = field(default_factory=dict)
     block_tables: Dict = field(default_factory=dict)   # cache group name -> [B, width] int32

@@ -44,7 +44,7 @@ class Engine:
         self.cache: Cache = model.new_cache(max_tokens, max_seqs, step_tokens=max_step_tokens)
         self.workspace = Workspace(model.device)
         self.steps_run = 0
-        self.use_graphs = use_graphs
+        self.use_graphs = use_graphs and model.graph_safe
         self.max_graph_batch = 256
         self._graphs: Dict[tuple, tuple] = {}
 
@@ -57,6 +57,17 @@ class Engine:
 
     def length(self, slot: int) -> int:
         return self.cache.length(slot)
+
+    def adopt_positions(self, slot: int, n: int) -> None:
+        """Lengthens a sequence by ``n`` positions without running tokens: the cache rows are
+        whatever the pages held.  For measurements that want decode steps at a given depth
+        without paying for the prompt; results of such a sequence mean nothing."""
+        new_len = self.cache.length(slot) + n
+        if new_len > self.model.spec.max_positions:
+            raise ContextOverflowError(f"sequence would reach {new_len} positions; the model has "
+                                       f"{self.model.spec.max_positions}")
+        self.cache.reserve([slot], [new_len])
+        self.cache.commit([slot], [new_len])
 
     # -- the step ------------------------------------------------------------------------
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
@@ -175,7 +186,7 @@ class Engine:
             step = StepContext(n_tokens=int(ids.size), n_seqs=len(slots), token_ids=d_ids, token_seq=d_seq,
                                token_pos=d_pos, cu_seqlens=d_cu, seq_lens=d_lens, seq_slots=d_slots,
                                max_new=max_new, max_len=int(lens.max()),
-                               total_q_tiles=sum((len(t) + 127) // 128 for t in tokens),
+                               new_counts=tuple(len(t) for t in tokens),
                                workspace=self.workspace)
             step.block_tables = block_tables
             step.want_rows = d_want if n_want else None

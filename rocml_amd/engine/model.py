@@ -10,7 +10,7 @@ from typing import Dict, List, Optional
 import torch
 
 from .. import ops
-from ..cache import Cache, CacheLineView, KVGroup
+from ..cache import Cache
 from ..cache.cache import HEADROOM_BYTES
 from ..config.spec import ModelSpec
 from ..errors import ConfigError
@@ -41,6 +41,9 @@ class DecoderModel:
         self.final_norm = build_norm(spec.final_norm, ctx)
         self.embed: Optional[torch.Tensor] = None
         self.lm_head: Optional[torch.Tensor] = None
+        # whether a decode step may be recorded as a graph: every part must say so
+        self.graph_safe = all(getattr(b, "graph_safe", True) for b in self.blocks) and \
+            getattr(self.final_norm, "graph_safe", True)
 
     # -- parameters --------------------------------------------------------------------
     def param_specs(self) -> Dict[str, ParamSpec]:
@@ -77,6 +80,37 @@ class DecoderModel:
                 n *= d
             total += n * torch.empty((), dtype=self.storage_dtype(p)).element_size()
         return total
+
+    def n_params(self) -> int:
+        total = 0
+        for p in self.param_specs().values():
+            n = 1
+            for d in p.shape:
+                n *= d
+            total += n
+        return total
+
+    def step_weight_bytes(self) -> int:
+        """Bytes of weights a step has to read once: every layer as often as the schedule runs
+        it and the output matrix; of the embedding table only the step's rows, which are not
+        counted (a tied table is read as the output matrix)."""
+        per_layer = []
+        for block in self.blocks:
+            n = 0
+            for p in block.param_specs().values():
+                e = 1
+                for d in p.shape:
+                    e *= d
+                n += e * torch.empty((), dtype=self.storage_dtype(p)).element_size()
+            per_layer.append(n)
+        size = torch.empty((), dtype=self.dtype).element_size()
+        return sum(per_layer[e.layer] for e in self.spec.schedule) + self.spec.vocab * self.spec.hidden * size
+
+    def step_flops(self, new_counts, starts, n_wanted: int) -> int:
+        """Floating-point operations of a step: the layers in schedule order and the output
+        product for the wanted rows."""
+        total = sum(self.blocks[e.layer].flops(new_counts, starts) for e in self.spec.schedule)
+        return total + 2 * n_wanted * self.spec.vocab * self.spec.hidden
 
     # -- cache -------------------------------------------------------------------------
     def cache_requests(self) -> List[Optional[object]]:
@@ -126,13 +160,11 @@ class DecoderModel:
             view = None
             if cache.has_line(owner):
                 group, line = cache.line(owner)
-                if isinstance(group, KVGroup):
-                    view = CacheLineView(group=group, line=line, k=group.k[line], v=group.v[line],
-                                         block_table=block_tables[group.name])
-                else:
-                    view = CacheLineView(group=group, line=line, state=group.state[line],
-                                         slots=step.seq_slots)
-            self.blocks[entry.layer].forward(step, x, view, owner == i)
+                view = group.view(line, step)
+            block = self.blocks[entry.layer]
+            if not getattr(block, "takes_pending", False):
+                ws.flush_pending()
+            block.forward(step, x, view, owner == i)
         if n_want == 0:
             ws.drop_pending()
             return None

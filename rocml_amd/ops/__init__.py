@@ -11,7 +11,7 @@ call raises.
 from __future__ import annotations
 
 import ctypes
-from typing import Dict, Optional
+from typing import Dict, Optional, Sequence
 
 import torch
 
@@ -41,7 +41,7 @@ _SIGNATURES = {
     },
     "attention": {
         "rocml_attention": [_P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I,
-                            _P, _I, _I, _I, _I, _I, _P, _LL, _P],
+                            _P, _I, _I, _P, _I, _I, _P, _LL, _P],
         "rocml_attention_decode_fused": [_P, _I, _I, _LL, _P, _P, _F, _P, _P, _I, _P, _P, _P, _P, _I, _P, _P,
                                          _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _LL, _P],
     },
@@ -295,12 +295,12 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache
               block_table: torch.Tensor, token_seq: torch.Tensor, token_pos: torch.Tensor,
               n_heads: int, n_kv_heads: int, head_dim: int, scale: float, window: Optional[int] = None,
               algo: int = ATTN_AUTO, workspace: Optional[torch.Tensor] = None,
-              cu_seqlens: Optional[torch.Tensor] = None, max_new: int = 0, total_q_tiles: int = 0,
-              max_len: int = 0, n_splits: int = 0) -> None:
+              cu_seqlens: Optional[torch.Tensor] = None, max_new: int = 0,
+              q_counts: Optional[Sequence[int]] = None, max_len: int = 0, n_splits: int = 0) -> None:
     """Attention of the step's query tokens over the cache.  Keys are ``[pages, Hkv, page, D]``,
-    values ``[pages, Hkv, D, page]``.  ``cu_seqlens``, ``max_new`` (most query tokens of a
-    sequence), ``total_q_tiles`` (sum of ceil(tokens / 128)) and ``max_len`` (longest context)
-    describe the step to the fast kernels; without them the plain kernel runs."""
+    values ``[pages, Hkv, D, page]``.  ``cu_seqlens`` (device), ``q_counts`` (the same knowledge on
+    the host: query tokens of each sequence), ``max_new`` (the most of them) and ``max_len``
+    (longest context) describe the step to the fast kernels; without them the plain kernel runs."""
     _dev(q, out, k_cache, v_cache, block_table, token_seq, token_pos, cu_seqlens)
     n_tokens = q.shape[0]
     if q.shape != (n_tokens, n_heads * head_dim) or out.shape != q.shape or out.dtype != q.dtype:
@@ -316,15 +316,20 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache
     if token_seq.numel() != n_tokens or token_pos.numel() != n_tokens:
         raise KernelError("one sequence index and one position per token are needed")
     n_seqs = 0
+    counts = None
     if cu_seqlens is not None:
         _want(cu_seqlens, torch.int32, "sequence offsets")
         n_seqs = cu_seqlens.numel() - 1
+        if q_counts is not None:
+            if len(q_counts) != n_seqs:
+                raise KernelError(f"{len(q_counts)} query counts for {n_seqs} sequences")
+            counts = (ctypes.c_int * n_seqs)(*[int(c) for c in q_counts])
     ws_ptr, ws_bytes = (None, 0) if workspace is None else (workspace.data_ptr(), workspace.numel() * workspace.element_size())
     _check("attention", library("attention").rocml_attention(
         _ptr(q), _ptr(out), _ptr(k_cache), _ptr(v_cache), _code(q), _ptr(block_table),
         block_table.shape[1], _ptr(token_seq), _ptr(token_pos), n_tokens, n_heads, n_kv_heads, head_dim,
         page, scale, 0 if window is None else int(window), algo, _ptr(cu_seqlens), n_seqs, max_new,
-        total_q_tiles, max_len, n_splits, ws_ptr, ws_bytes, _stream()))
+        counts, max_len, n_splits, ws_ptr, ws_bytes, _stream()))
 
 
 FUSED_DECODE_HEAD_DIMS = (64, 128, 192, 256)

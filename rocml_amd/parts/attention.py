@@ -22,11 +22,16 @@ from .registry import build_position, register_mixer
 
 
 class Attention(Mixer):
+    adds_only = True
+
     def __init__(self, spec: AttentionSpec, ctx: BuildContext):
         if spec.n_heads % spec.n_kv_heads != 0:
             raise ConfigError(f"{spec.n_heads} query heads are not a multiple of {spec.n_kv_heads} key/value heads")
         if spec.qk_norm is not None and spec.qk_norm.size != spec.head_dim:
             raise ConfigError("the per-head norm must span the head size")
+        if spec.qk_norm is not None and spec.qk_norm.kind != "rmsnorm":
+            # the norm of q and k runs inside the rotation and attention kernels, which know one kind
+            raise ConfigError(f"the per-head norm must be of kind 'rmsnorm', got {spec.qk_norm.kind!r}")
         if spec.window is not None and spec.window <= 0:
             raise ConfigError(f"window must be positive, got {spec.window}")
         self.spec = spec
@@ -59,6 +64,17 @@ class Attention(Mixer):
         if self.spec.qk_norm is not None:
             self.q_gain = tensors["q_norm.weight"]
             self.k_gain = tensors["k_norm.weight"]
+
+    def flops(self, new_counts, starts) -> int:
+        # the products with the weights, and 4 * heads * head size per query and key it sees
+        keys = 0
+        w = self.spec.window
+        for n, s0 in zip(new_counts, starts):
+            if w is None:
+                keys += n * s0 + n * (n + 1) // 2
+            else:
+                keys += sum(min(s0 + i + 1, w) for i in range(n))
+        return 2 * sum(new_counts) * self.matrix_elements() + 4 * self.spec.n_heads * self.spec.head_dim * keys
 
     def activation_bytes(self, n_tokens: int) -> int:
         size = 2 if self.dtype == torch.bfloat16 else 4
@@ -111,7 +127,7 @@ class Attention(Mixer):
                                     step.token_pos, write_kv=owns_cache, n_splits=max(splits, 1))
             ops.attention(q, o, cache.k, cache.v, cache.block_table, step.token_seq, step.token_pos,
                           s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, workspace=ws.scratch(),
-                          cu_seqlens=step.cu_seqlens, max_new=step.max_new, total_q_tiles=step.total_q_tiles,
+                          cu_seqlens=step.cu_seqlens, max_new=step.max_new, q_counts=step.new_counts,
                           max_len=step.max_len, n_splits=self._decode_splits(step, cache))
         splits = ops.gemm(o, self.w_o, x_accum, accumulate=True, workspace=ws.scratch(), defer=True)
         if splits:

@@ -15,8 +15,11 @@ layer is assembled from parts that know nothing about the model around them:
 Mixers and feed-forwards add their result into the 32-bit residual stream they are
 handed (``x_accum``), which lets a product's epilogue do the residual sum.  A part whose
 last product was split along K may leave the final addition of the partial sums to the
-norm that reads ``x_accum`` next (``step.workspace.set_pending``); whoever reads
-``x_accum`` in another way calls ``step.workspace.flush_pending()`` first.
+norm that reads ``x_accum`` next (``step.workspace.set_pending``).  Nobody else has to know:
+the stream is completed (``flush_pending``) before it is handed to a norm that cannot add the
+sums itself (no ``fuses_pending``), to a mixer or feed-forward that does not declare
+``adds_only`` (that it only ever adds into ``x_accum`` and never reads it), and to a block
+arrangement that does not declare ``takes_pending``.
 """
 from __future__ import annotations
 
@@ -62,12 +65,33 @@ class StateRequest:
 
 
 class Part:
+    # False: forward() waits for the GPU or works on the host (reads a tensor back, loops over
+    # tokens), so a decode step with this part cannot be recorded and replayed as a graph
+    graph_safe = True
+
     def param_specs(self) -> Dict[str, ParamSpec]:
         return {}
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         """Receives the tensors named by ``param_specs``, already on the device and in
         the type their role asks for."""
+
+    def matrix_elements(self) -> int:
+        """Elements of the part's matrices (what a step multiplies each token with)."""
+        total = 0
+        for p in self.param_specs().values():
+            if p.role == "matrix":
+                n = 1
+                for d in p.shape:
+                    n *= d
+                total += n
+        return total
+
+    def flops(self, new_counts, starts) -> int:
+        """Floating-point operations of a step in which sequence ``b`` brings ``new_counts[b]``
+        tokens on top of ``starts[b]`` cached ones: two per token and matrix element unless the
+        part knows better."""
+        return 2 * sum(new_counts) * self.matrix_elements()
 
     def activation_bytes(self, n_tokens: int) -> int:
         """Bytes of workspace buffers the part asks for in a step of ``n_tokens`` tokens; what
@@ -76,6 +100,8 @@ class Part:
 
 
 class Norm(Part):
+    fuses_pending = False     # True: forward() takes ``pending`` partial sums and adds them to x itself
+
     def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
         raise NotImplementedError
 
@@ -93,6 +119,8 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    adds_only = False     # True: forward() never reads x_accum, it only adds into it
+
     def cache_request(self) -> Optional[Any]:
         return None
 
@@ -105,5 +133,7 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    adds_only = False     # True: forward() never reads x_accum, it only adds into it
+
     def forward(self, step: Any, xn: torch.Tensor, x_accum: torch.Tensor) -> None:
         raise NotImplementedError

@@ -26,6 +26,7 @@ class PreNormBlock(Part):
         self.mixer = self.children["mixer"]
         self.ffn_norm = self.children["ffn_norm"]
         self.ffn = self.children["ffn"]
+        self.graph_safe = all(getattr(c, "graph_safe", True) for c in self.children.values())
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         return {f"{name}.{p}": spec for name, child in self.children.items()
@@ -39,15 +40,25 @@ class PreNormBlock(Part):
     def cache_request(self):
         return self.mixer.cache_request()
 
+    def flops(self, new_counts, starts) -> int:
+        return self.mixer.flops(new_counts, starts) + self.ffn.flops(new_counts, starts)
+
     def activation_bytes(self, n_tokens: int) -> int:
         size = 2 if self.dtype == torch.bfloat16 else 4
         return n_tokens * self.hidden * size + self.mixer.activation_bytes(n_tokens) + self.ffn.activation_bytes(n_tokens)
 
+    takes_pending = True      # forward() may be handed a stream that still lacks deferred sums
+
     def forward(self, step, x: torch.Tensor, cache, owns_cache: bool) -> None:
-        xn = step.workspace.get("block.xn", tuple(x.shape), self.dtype)
+        ws = step.workspace
+        xn = ws.get("block.xn", tuple(x.shape), self.dtype)
         self._norm(step, self.mixer_norm, x, xn)
+        if not getattr(self.mixer, "adds_only", False):
+            ws.flush_pending()
         self.mixer.forward(step, xn, x, cache, owns_cache)
         self._norm(step, self.ffn_norm, x, xn)
+        if not getattr(self.ffn, "adds_only", False):
+            ws.flush_pending()
         self.ffn.forward(step, xn, x)
 
     @staticmethod

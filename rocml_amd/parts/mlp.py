@@ -16,6 +16,8 @@ from .registry import register_feed_forward
 
 
 class GatedMlp(FeedForward):
+    adds_only = True
+
     def __init__(self, spec: GatedMlpSpec, ctx: BuildContext):
         if spec.activation != "silu":
             raise ConfigError(f"activation {spec.activation!r} is not supported (silu only)")

@@ -110,9 +110,10 @@ def random_tensors(param_specs: Dict[str, ParamSpec], names: Dict[str, str], see
 
 
 def write_model_dir(path: str, config: Dict, seed: int, dtype: torch.dtype = torch.bfloat16,
-                    norm_jitter: bool = True) -> str:
+                    norm_jitter: bool = True, device="cpu") -> str:
     """Writes ``config.json`` and ``model.safetensors`` for ``config`` (config.json's
-    dictionary) with random weights; returns ``path``."""
+    dictionary) with random weights; returns ``path``.  ``device`` is where the values are
+    drawn (they are the same anywhere; a GPU draws a large model in seconds)."""
     from safetensors.torch import save_file
     from ..config import architecture_of
     from ..engine.model import DecoderModel
@@ -121,7 +122,7 @@ def write_model_dir(path: str, config: Dict, seed: int, dtype: torch.dtype = tor
     spec = arch.to_spec(cfg)
     model = DecoderModel(spec, torch.float32, device="meta")
     names = arch.checkpoint_names(spec)
-    tensors = dict(random_tensors(model.param_specs(), names, seed, dtype, norm_jitter))
+    tensors = {name: t.cpu() for name, t in random_tensors(model.param_specs(), names, seed, dtype, norm_jitter, device)}
     os.makedirs(path, exist_ok=True)
     with open(os.path.join(path, "config.json"), "w", encoding="utf-8") as f:
         json.dump(cfg.to_dict() if hasattr(cfg, "to_dict") else config, f, indent=2)

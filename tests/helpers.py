@@ -97,6 +97,14 @@ def rel_to_max(got: torch.Tensor, ref: torch.Tensor) -> float:
     return float((got.to(torch.float64) - ref).abs().max() / ref.abs().max())
 
 
+def per_position(got: torch.Tensor, ref: torch.Tensor) -> float:
+    """The worst position's largest absolute difference over that position's largest absolute
+    reference value: a fault at one place is not hidden by large logits elsewhere."""
+    ref = ref.to(torch.float64)
+    diff = (got.to(torch.float64) - ref).abs().amax(dim=-1)
+    return float((diff / ref.abs().amax(dim=-1)).max())
+
+
 def run_whole(engine, tokens: Sequence[int]) -> torch.Tensor:
     """One request alone, whole: logits at every position, [T, V] on the CPU."""
     from rocml_amd.engine import StepEntry

@@ -56,8 +56,17 @@ def rope_neox(x: torch.Tensor, positions: Sequence[int], theta: float) -> torch.
     return out
 
 
+def _same(t: torch.Tensor) -> torch.Tensor:
+    return t
+
+
+def round_bfloat16(t: torch.Tensor) -> torch.Tensor:
+    """The nearest bfloat16 value (ties to even), kept in the tensor's own type."""
+    return t.to(torch.bfloat16).to(t.dtype)
+
+
 def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
-                     scale: float, window: Optional[int] = None) -> torch.Tensor:
+                     scale: float, window: Optional[int] = None, rounded=_same) -> torch.Tensor:
     """Causal softmax attention of one whole sequence with grouped heads.
 
     ``q`` is ``[T, Hq, D]``, ``k`` and ``v`` are ``[T, Hkv, D]``.  Query head
@@ -67,7 +76,10 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     (rocml-kernels/kernels/attn_prefill.hip:121,167-190); ``out = softmax(s) @ v``
     (rocml-kernels/kernels/attn_decode.hip:227-254 give the same sum after merging).
     ``window`` (not in the reference, which has full attention only) restricts
-    the keys to the last ``window`` positions ``[p - window + 1, p]``."""
+    the keys to the last ``window`` positions ``[p - window + 1, p]``.
+    ``rounded`` is applied to the unnormalised probabilities ``e^(s - max)`` that multiply the
+    values; their sum, which divides the result, is taken before rounding (a low-precision
+    second product with full-precision statistics)."""
     t_len, hq, d = q.shape
     hkv = k.shape[1]
     group = hq // hkv
@@ -78,8 +90,7 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
             lo = 0 if window is None else max(0, p - window + 1)
             scores = (k[lo:p + 1, kv] @ q[p, h]) * scale
             e = torch.exp(scores - scores.max())
-            prob = e / e.sum()
-            out[p, h] = prob @ v[lo:p + 1, kv]
+            out[p, h] = (rounded(e) @ v[lo:p + 1, kv]) / e.sum()
     return out
 
 
@@ -95,12 +106,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
 
 
 def attention_block(x: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, cfg: dict,
-                    positions: Sequence[int], window: Optional[int]) -> torch.Tensor:
+                    positions: Sequence[int], window: Optional[int], rounded=_same) -> torch.Tensor:
     """One layer's attention sub-block on the normalised input
     (rocml/src/forward/attention_chunk.rs:97-256,316-330): three projections
     without bias, per-head RMSNorm of q and k with one ``[D]`` gain each and the
     model's eps, rotary embedding of q and k, causal attention with
-    ``scale = 1/sqrt(D)`` (rocml/src/forward/attention.rs:160), output projection."""
+    ``scale = 1/sqrt(D)`` (rocml/src/forward/attention.rs:160), output projection.
+    ``rounded`` is applied where a low-precision engine stores a tensor: q, k and v as the
+    attention reads them, the probabilities, and the attention's output."""
     hq = cfg["num_attention_heads"]
     hkv = cfg["num_key_value_heads"]
     d = cfg["head_dim"]
@@ -111,18 +124,19 @@ def attention_block(x: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, cf
     v = linear(x, w[prefix + "self_attn.v_proj.weight"]).reshape(t_len, hkv, d)
     q = rmsnorm(q, w[prefix + "self_attn.q_norm.weight"], eps)
     k = rmsnorm(k, w[prefix + "self_attn.k_norm.weight"], eps)
-    q = rope_neox(q, positions, cfg["rope_theta"])
-    k = rope_neox(k, positions, cfg["rope_theta"])
-    o = causal_attention(q, k, v, 1.0 / math.sqrt(d), window)
+    q = rounded(rope_neox(q, positions, cfg["rope_theta"]))
+    k = rounded(rope_neox(k, positions, cfg["rope_theta"]))
+    o = rounded(causal_attention(q, k, rounded(v), 1.0 / math.sqrt(d), window, rounded))
     return linear(o.reshape(t_len, hq * d), w[prefix + "self_attn.o_proj.weight"])
 
 
-def mlp_block(x: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str) -> torch.Tensor:
+def mlp_block(x: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, rounded=_same) -> torch.Tensor:
     """Gated feed-forward on the normalised input
-    (rocml/src/forward/ffn.rs:36-107): ``down(silu(gate(x)) * up(x))``."""
+    (rocml/src/forward/ffn.rs:36-107): ``down(silu(gate(x)) * up(x))``; ``rounded`` is
+    applied to the gated activation, the one tensor a low-precision engine stores here."""
     g = linear(x, w[prefix + "mlp.gate_proj.weight"])
     u = linear(x, w[prefix + "mlp.up_proj.weight"])
-    return linear(swiglu(g, u), w[prefix + "mlp.down_proj.weight"])
+    return linear(rounded(swiglu(g, u)), w[prefix + "mlp.down_proj.weight"])
 
 
 def layer_windows(cfg: dict) -> List[Optional[int]]:
@@ -138,7 +152,8 @@ def layer_windows(cfg: dict) -> List[Optional[int]]:
 
 
 def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: Sequence[int],
-            dtype: torch.dtype = torch.float64, first_position: int = 0) -> torch.Tensor:
+            dtype: torch.dtype = torch.float64, first_position: int = 0, rounded=_same,
+            last: Optional[int] = None) -> torch.Tensor:
     """Logits ``[T, V]`` at every position of one whole sequence.
 
     Pre-norm residual blocks (rocml/src/forward/chunk_forward.rs:96-135):
@@ -146,19 +161,25 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: Sequence[int],
     the output matrix, which is the embedding table when the checkpoint has no
     ``lm_head.weight`` (rocml/src/weights/mod.rs:48-62,
     rocml/src/forward/mod.rs:342-380).  ``first_position`` shifts every position
-    (used by the shift-invariance test only)."""
-    w = {name: t.to(dtype) for name, t in weights.items()}
+    (used by the shift-invariance test only).  ``rounded`` (``round_bfloat16`` for the oracle
+    of a bfloat16 engine) is applied to every tensor such an engine holds in low precision:
+    the matrices, the normalised activations that feed a product, q, k, v, the probabilities,
+    the attention's output and the gated activation; the residual stream, the norms'
+    statistics, the rotation, the softmax statistics and all sums stay in ``dtype``."""
+    w = {name: (rounded(t.to(dtype)) if t.dim() > 1 else t.to(dtype)) for name, t in weights.items()}
     eps = cfg["rms_norm_eps"]
     positions = [first_position + t for t in range(len(tokens))]
     windows = layer_windows(cfg)
     x = embedding(w["model.embed_tokens.weight"], tokens)
     for layer in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{layer}."
-        xn = rmsnorm(x, w[p + "input_layernorm.weight"], eps)
-        x = x + attention_block(xn, w, p, cfg, positions, windows[layer])
-        xn = rmsnorm(x, w[p + "post_attention_layernorm.weight"], eps)
-        x = x + mlp_block(xn, w, p)
-    xn = rmsnorm(x, w["model.norm.weight"], eps)
+        xn = rounded(rmsnorm(x, w[p + "input_layernorm.weight"], eps))
+        x = x + attention_block(xn, w, p, cfg, positions, windows[layer], rounded)
+        xn = rounded(rmsnorm(x, w[p + "post_attention_layernorm.weight"], eps))
+        x = x + mlp_block(xn, w, p, rounded)
+    if last is not None:            # logits of the last positions only (a large vocabulary)
+        x = x[-last:]
+    xn = rounded(rmsnorm(x, w["model.norm.weight"], eps))
     head = w["lm_head.weight"] if "lm_head.weight" in w else w["model.embed_tokens.weight"]
     return linear(xn, head)
 

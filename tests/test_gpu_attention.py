@@ -75,7 +75,7 @@ def _run(dev, seqs, hq, hkv, d, scale, window, algo, n_splits=0):
     ws = torch.empty(32 << 20, dtype=torch.uint8, device="cuda")
     ops.attention(dev["q"], out, dev["kc"], dev["vc"], dev["table"], dev["tok_seq"], dev["tok_pos"], hq, hkv,
                   d, scale, window, algo=algo, workspace=ws, cu_seqlens=dev["cu"],
-                  max_new=max(n for _, n in seqs), total_q_tiles=sum((n + 127) // 128 for _, n in seqs),
+                  max_new=max(n for _, n in seqs), q_counts=[n for _, n in seqs],
                   max_len=max(length for length, _ in seqs), n_splits=n_splits)
     return out.cpu()
 
@@ -210,7 +210,7 @@ def _fused_case(seqs, hq, hkv, d, qkv_splits, attn_splits, window, seed, norm=Tr
                             d if rotate else 0, q_dev, kc2, vc2, dev["table"], dev["tok_seq"], dev["tok_pos"],
                             n_splits=qkv_splits)
     ops.attention(q_dev, out2, kc2, vc2, dev["table"], dev["tok_seq"], dev["tok_pos"], hq, hkv, d, scale, window,
-                  algo=MFMA, workspace=ws, cu_seqlens=dev["cu"], max_new=1, total_q_tiles=n, max_len=max_len,
+                  algo=MFMA, workspace=ws, cu_seqlens=dev["cu"], max_new=1, q_counts=[1] * n, max_len=max_len,
                   n_splits=attn_splits)
     out = torch.full_like(q_dev, float("nan"))
     kc3, vc3 = dev["kc"].clone(), dev["vc"].clone()

@@ -114,3 +114,59 @@ def test_refused_steps_leave_the_engine_as_it_was(models):
     engine.cache.check()
     got = engine.step([StepEntry(a, toks[60:], list(range(40)))]).cpu()    # goes on as if nothing had happened
     assert helpers.rel_to_max(got, ref[60:]) < TOL["float32"]
+
+
+# Against an oracle that rounds to bfloat16 exactly where the engine does (matrices, normalised
+# activations, q, cached k and v, probabilities, attention output, gated activation), what is left
+# is the order of sums and the probabilities' rounding relative to another running maximum; the
+# bound holds for every position on its own, so one bad place cannot hide behind large logits.
+ROUNDED_TOL = 4e-3
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "G", "H"])
+def test_bfloat16_against_an_oracle_that_rounds_where_the_engine_does(models, name):
+    path, cfg, weights = models[name]
+    engine = _engine(path, "bfloat16")
+    prompts = [helpers.random_tokens(n, cfg["vocab_size"], 300 + i) for i, n in enumerate(LENGTHS[name])]
+    refs = [plain.forward(cfg, weights, p, rounded=plain.round_bfloat16) for p in prompts]
+    for p, ref in zip(prompts, refs):
+        assert helpers.per_position(helpers.run_whole(engine, p), ref) < ROUNDED_TOL, f"whole, length {len(p)}"
+        assert helpers.per_position(helpers.run_tail_by_one(engine, p, 32), ref) < ROUNDED_TOL, f"tail, length {len(p)}"
+    got = helpers.run_batch(engine, prompts, [max(1, len(p) - 3 * (j + 1)) for j, p in enumerate(prompts)])
+    for g, ref in zip(got, refs):
+        assert helpers.per_position(g, ref) < ROUNDED_TOL
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,n_seqs", [("H", 33), ("H", 64), ("F", 33), ("F", 64)])
+def test_many_sequences_in_a_step(models, name, dtype, n_seqs):
+    """33 and 64 sequences of unequal lengths: their prompts in one step, then decode steps in
+    which the shorter requests end one after the other, so the batch shrinks through the row
+    counts the few-rows kernels are built for; then the same slots again with every sequence
+    decoding side by side, the steps recorded once and replayed.  H takes the decode attention
+    that reads the projection itself, F is wide enough for products cut along K."""
+    from rocml_amd.engine import StepEntry
+    path, cfg, weights = models[name]
+    engine = _engine(path, dtype, max_tokens=64 * 4 * n_seqs)
+    oracle_w = _oracle_weights(weights, dtype)
+    lengths = [10 + (7 * i) % 90 for i in range(n_seqs)]
+    tails = [1 + i % 8 for i in range(n_seqs)]                  # tokens fed one by one after the prompt
+    seqs = [helpers.random_tokens(n + t, cfg["vocab_size"], 500 + i) for i, (n, t) in enumerate(zip(lengths, tails))]
+    refs = [plain.forward(cfg, oracle_w, s) for s in seqs]
+    got = helpers.run_batch(engine, seqs, lengths)
+    worst = max(helpers.rel_to_max(g, r) for g, r in zip(got, refs))
+    assert worst < TOL[dtype], f"{n_seqs} sequences: {worst}"
+    engine.cache.check()
+    assert not engine.cache.lengths
+    slots = [engine.new_sequence() for _ in seqs]
+    engine.step([StepEntry(s, q[:5], []) for s, q in zip(slots, seqs)])
+    for k in range(5, 10):
+        logits = engine.step([StepEntry(s, [q[k]], [0]) for s, q in zip(slots, seqs)]).cpu()
+        expect = torch.stack([r[k] for r in refs])
+        assert helpers.rel_to_max(logits, expect) < TOL[dtype], f"decode step {k}"
+    recorded = [key for key, entry in engine._graphs.items() if entry[1] is not None]
+    assert engine.use_graphs and any(key[0] == n_seqs for key in recorded)
+    for s in slots:
+        engine.release(s)
+    engine.cache.check()

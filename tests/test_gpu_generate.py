@@ -170,3 +170,93 @@ def test_position_and_reset_through_the_entry_point(models):
     c = model.new_sequence()                       # a slot and pages that were just given back, not cleared
     got = model.step([StepEntry(c, toks, list(range(20)))]).cpu()
     assert model.position(c) == 20 and helpers.rel_to_max(got, ref) < 2e-5
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 2e-2)])
+def test_prompts_far_longer_than_the_window_through_the_entry_point(models, dtype, tol):
+    """Config D has layers with a window of 70.  With ``max_batch`` set, their cache group is
+    sized for its windows, not for whole sequences; a prompt of 1,000 tokens passes through it in
+    pieces, and generation continues from what the window still holds."""
+    from rocml_amd.api import LoadOptions, Model
+    from rocml_amd.engine import Engine, StepEntry
+    from rocml_amd.weights import load_model
+    path, cfg, weights = models["D"]
+    w = weights if dtype == "float32" else {k: (v if v.dim() == 1 else v.to(torch.bfloat16).float()) for k, v in weights.items()}
+    long_prompt = helpers.random_tokens(1000, cfg["vocab_size"], 91)
+    short_prompt = helpers.random_tokens(300, cfg["vocab_size"], 92)
+    model = Model.load(path, LoadOptions(dtype=dtype, ctx=1100, max_batch=2))
+    windowed = [g for g in model.engine.cache.kv_groups if g.window is not None][0]
+    full = [g for g in model.engine.cache.kv_groups if g.window is None][0]
+    assert windowed.n_pages < full.n_pages
+    got = model.generate([long_prompt, short_prompt], max_new_tokens=6)
+    want = [plain.greedy(cfg, w, p, 6) for p in (long_prompt, short_prompt)]
+    for g, wt, p in zip(got, want, (long_prompt, short_prompt)):
+        if dtype == "float32":
+            assert g.tokens == wt
+        elif g.tokens != wt:
+            k = next(i for i in range(6) if g.tokens[i] != wt[i])
+            assert near_tie(cfg, w, p, wt, k)
+    model.engine.cache.check()
+    assert not model.engine.cache.lengths
+    # logits, with pieces far smaller than the prompt: the windowed group is then a handful of pages
+    engine = Engine(load_model(path, dtype=dtype, device="cuda:0"), max_tokens=2 * 1100, max_seqs=2, max_step_tokens=96)
+    windowed = [g for g in engine.cache.kv_groups if g.window is not None][0]
+    assert windowed.n_pages == 2 * 4 + 2
+    ref = plain.forward(cfg, w, long_prompt)
+    a, b = engine.new_sequence(), engine.new_sequence()
+    places = [0, 69, 70, 71, 500, 998, 999]
+    logits = engine.step([StepEntry(a, long_prompt[:999], places[:-1]), StepEntry(b, short_prompt[:10], [])]).cpu()
+    assert helpers.rel_to_max(logits, ref[places[:-1]]) < tol
+    logits = engine.step([StepEntry(a, [long_prompt[999]], [0]), StepEntry(b, [short_prompt[10]], [])]).cpu()
+    assert helpers.rel_to_max(logits, ref[999:]) < tol
+    engine.release(a)
+    engine.release(b)
+    engine.cache.check()
+
+
+def test_generation_stops_at_the_models_end_of_sequence_id(models, tmp_path):
+    """``eos_token_id`` of config.json (or generation_config.json) ends a sequence by default and
+    is not emitted; ``ignore_eos`` and the command line's --ignore-eos go on."""
+    import json
+    import shutil
+    from rocml_amd.cli import main
+    path, cfg, weights = models["B"]
+    prompt = helpers.random_tokens(9, cfg["vocab_size"], 7)
+    free = plain.greedy(cfg, weights, prompt, 8)
+    eos = free[3]
+    cut = free[:free.index(eos)]
+    with_eos = str(tmp_path / "with_eos")
+    shutil.copytree(path, with_eos)
+    with open(f"{with_eos}/config.json", "w") as f:
+        json.dump(dict(cfg, eos_token_id=eos), f)
+    model = _load(with_eos, "float32", ctx=64, max_batch=1)
+    r = model.generate([prompt], max_new_tokens=8)[0]
+    assert r.tokens == cut and r.finish_reason == "stop"
+    assert model.generate([prompt], max_new_tokens=8, ignore_eos=True)[0].tokens == free
+    in_generation_config = str(tmp_path / "generation_config")
+    shutil.copytree(path, in_generation_config)
+    with open(f"{in_generation_config}/generation_config.json", "w") as f:
+        json.dump({"eos_token_id": [eos, free[6]]}, f)
+    model = _load(in_generation_config, "float32", ctx=64, max_batch=1)
+    assert model.generate([prompt], max_new_tokens=8)[0].tokens == cut
+    assert _load(path, "float32", ctx=64, max_batch=1).generate([prompt], max_new_tokens=8)[0].tokens == free
+
+
+def test_a_catalog_model_has_the_weights_its_written_folder_has(tmp_path):
+    """``--model tiny-b`` draws its weights on the GPU, ``init`` writes them on the CPU: the same
+    seed gives the same bits, so both generate the same tokens and hold the same tensors."""
+    from rocml_amd.api import Model
+    from rocml_amd.cli import main
+    out = str(tmp_path / "tiny_b")
+    assert main(["init", "--model", "tiny-b", "--out", out, "--weights-seed", "5", "--dtype", "float32"]) == 0
+    by_name = Model.load("tiny-b", dtype="float32", seed=5, ctx=64, max_batch=2)
+    from_folder = Model.load(out, dtype="float32", ctx=64, max_batch=2)
+    a, b = by_name.engine.model, from_folder.engine.model
+    assert torch.equal(a.embed, b.embed) and torch.equal(a.lm_head, b.lm_head)
+    for x, y in zip(a.blocks, b.blocks):
+        assert torch.equal(x.mixer.w_qkv, y.mixer.w_qkv) and torch.equal(x.ffn.w_down, y.ffn.w_down)
+        assert torch.equal(x.mixer.q_gain, y.mixer.q_gain) and torch.equal(x.mixer_norm.gain, y.mixer_norm.gain)
+    prompts = [[3, 17, 200], [5, 6, 7, 8, 9, 10, 11]]
+    assert [r.tokens for r in by_name.generate(prompts, max_new_tokens=6)] == \
+        [r.tokens for r in from_folder.generate(prompts, max_new_tokens=6)]
+    assert not torch.equal(Model.load("tiny-b", dtype="float32", seed=6, ctx=64).engine.model.embed, a.embed)

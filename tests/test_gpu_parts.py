@@ -146,7 +146,7 @@ def test_norm_rope_and_mlp_parts_alone():
     ffn.bind({n: t.cuda() for n, t in ws.items()})
     pos = torch.tensor([5, 6, 7, 0, 1, 2, 3, 4, 900], dtype=torch.int32).cuda()
     step = StepContext(n_tokens=9, n_seqs=1, token_ids=pos, token_seq=pos, token_pos=pos, cu_seqlens=pos, seq_lens=pos,
-                       seq_slots=pos, max_new=9, max_len=9, total_q_tiles=1, workspace=Workspace("cuda:0"))
+                       seq_slots=pos, max_new=9, max_len=9, new_counts=(9,), workspace=Workspace("cuda:0"))
     acc = x.cuda().clone()
     ffn.forward(step, x.cuda(), acc)
     step.workspace.flush_pending()                                       # a part may leave its last sum to the next norm
@@ -176,6 +176,7 @@ def _toy_parts():
     class DecayMixer(Mixer):
         """state <- decay * state + W_in x, out = W_out state: a running sum per sequence,
         kept in the cache's fixed-size state and advanced once per token, in order."""
+        graph_safe = False        # loops over tokens on the host
 
         def __init__(self, spec, ctx):
             self.spec = spec
@@ -207,7 +208,8 @@ def test_toy_mixer_with_state_registers_builds_and_steps():
     toy = _block(32, DecaySpec(32, 12, 0.9))
     att = _block(32, _attention_spec(32, 2, 1, 16))
     spec = _spec([toy, att, toy], [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2)], 32, 77)
-    engine, w = _engine(spec, "float32", seed=5, use_graphs=False)
+    engine, w = _engine(spec, "float32", seed=5)
+    assert not engine.use_graphs                                 # a part of the model said it cannot be recorded
     assert len(engine.cache.state_groups) == 1 and engine.cache.state_groups[0].n_lines == 2
 
     def reference(tokens):
@@ -264,6 +266,7 @@ def _toy_routed_and_position():
     class RoutedFfn(FeedForward):
         """Router logits in 32-bit, the best ``top_k`` experts per token weighted by a softmax over
         their logits, each expert a small SwiGLU; tokens are gathered per expert."""
+        graph_safe = False        # the gathers have sizes that depend on the routing
 
         def __init__(self, spec, ctx):
             self.spec = spec
@@ -326,7 +329,7 @@ def test_toy_routed_feed_forward_and_toy_position_encoding():
         return BlockSpec(mixer=mixer, ffn=ffn, mixer_norm=NormSpec(hidden, 1e-5), ffn_norm=NormSpec(hidden, 1e-5))
     layers = [block(att_slow, routed), _block(hidden, _attention_spec(hidden, 4, 2, d)), block(att_slow, routed)]
     spec = _spec(layers, [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2)], hidden, 83)
-    engine, w = _engine(spec, "float32", seed=8, use_graphs=False)
+    engine, w = _engine(spec, "float32", seed=8)
 
     def rope_slow(x, positions):
         return plain.rope_neox(x, [p / slow.factor for p in positions], slow.theta)
