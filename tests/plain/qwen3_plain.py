@@ -106,14 +106,15 @@ def linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
 
 
 def attention_block(x: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, cfg: dict,
-                    positions: Sequence[int], window: Optional[int], rounded=_same) -> torch.Tensor:
+                    positions: Sequence[int], window: Optional[int], rounded=_same, rounded_probs=None) -> torch.Tensor:
     """One layer's attention sub-block on the normalised input
     (rocml/src/forward/attention_chunk.rs:97-256,316-330): three projections
     without bias, per-head RMSNorm of q and k with one ``[D]`` gain each and the
     model's eps, rotary embedding of q and k, causal attention with
     ``scale = 1/sqrt(D)`` (rocml/src/forward/attention.rs:160), output projection.
     ``rounded`` is applied where a low-precision engine stores a tensor: q, k and v as the
-    attention reads them, the probabilities, and the attention's output."""
+    attention reads them and the attention's output; ``rounded_probs`` (the same unless given)
+    to the probabilities, which only an engine whose second product runs in low precision rounds."""
     hq = cfg["num_attention_heads"]
     hkv = cfg["num_key_value_heads"]
     d = cfg["head_dim"]
@@ -126,7 +127,8 @@ def attention_block(x: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, cf
     k = rmsnorm(k, w[prefix + "self_attn.k_norm.weight"], eps)
     q = rounded(rope_neox(q, positions, cfg["rope_theta"]))
     k = rounded(rope_neox(k, positions, cfg["rope_theta"]))
-    o = rounded(causal_attention(q, k, rounded(v), 1.0 / math.sqrt(d), window, rounded))
+    o = rounded(causal_attention(q, k, rounded(v), 1.0 / math.sqrt(d), window,
+                                 rounded if rounded_probs is None else rounded_probs))
     return linear(o.reshape(t_len, hq * d), w[prefix + "self_attn.o_proj.weight"])
 
 
@@ -153,7 +155,7 @@ def layer_windows(cfg: dict) -> List[Optional[int]]:
 
 def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: Sequence[int],
             dtype: torch.dtype = torch.float64, first_position: int = 0, rounded=_same,
-            last: Optional[int] = None) -> torch.Tensor:
+            last: Optional[int] = None, rounded_probs=None) -> torch.Tensor:
     """Logits ``[T, V]`` at every position of one whole sequence.
 
     Pre-norm residual blocks (rocml/src/forward/chunk_forward.rs:96-135):
@@ -165,7 +167,9 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: Sequence[int],
     of a bfloat16 engine) is applied to every tensor such an engine holds in low precision:
     the matrices, the normalised activations that feed a product, q, k, v, the probabilities,
     the attention's output and the gated activation; the residual stream, the norms'
-    statistics, the rotation, the softmax statistics and all sums stay in ``dtype``."""
+    statistics, the rotation, the softmax statistics and all sums stay in ``dtype``.
+    ``rounded_probs`` replaces it for the probabilities alone (``lambda t: t`` for an engine
+    whose attention multiplies probabilities and values in full precision)."""
     w = {name: (rounded(t.to(dtype)) if t.dim() > 1 else t.to(dtype)) for name, t in weights.items()}
     eps = cfg["rms_norm_eps"]
     positions = [first_position + t for t in range(len(tokens))]
@@ -174,7 +178,7 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: Sequence[int],
     for layer in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{layer}."
         xn = rounded(rmsnorm(x, w[p + "input_layernorm.weight"], eps))
-        x = x + attention_block(xn, w, p, cfg, positions, windows[layer], rounded)
+        x = x + attention_block(xn, w, p, cfg, positions, windows[layer], rounded, rounded_probs)
         xn = rounded(rmsnorm(x, w[p + "post_attention_layernorm.weight"], eps))
         x = x + mlp_block(xn, w, p, rounded)
     if last is not None:            # logits of the last positions only (a large vocabulary)

@@ -117,18 +117,42 @@ def test_refused_steps_leave_the_engine_as_it_was(models):
 
 
 # Against an oracle that rounds to bfloat16 exactly where the engine does (matrices, normalised
-# activations, q, cached k and v, probabilities, attention output, gated activation), what is left
-# is the order of sums and the probabilities' rounding relative to another running maximum; the
-# bound holds for every position on its own, so one bad place cannot hide behind large logits.
-ROUNDED_TOL = 4e-3
+# activations, q, cached k and v, probabilities, attention output, gated activation), the engine's
+# logits are the oracle's to seven digits, until one value lies so close to the middle between two
+# bfloat16 numbers that 32-bit and 64-bit arithmetic round it to different sides; that one step
+# of the type spreads through every later rounded tensor and the difference becomes the noise of
+# the type (a few thousandths of the largest logit).  A sequence of one to four tokens has so few
+# rounded values that most stay clear of it.  So:
+#  * of twelve whole prompts of one to four tokens most must agree to 1e-5 (measured 1e-7): a
+#    tensor rounded in another place, or not rounded, or a constant that is off, fails all of them;
+#  * every position of every way of cutting stays within 1e-2 of its own largest logit.
+# Head sizes that run the plain attention kernel (A, C, E) multiply probabilities and values in
+# 32-bit, so their oracle leaves the probabilities alone, and their decode steps, which cut the
+# keys as a prompt does, agree like whole prompts; the matrix-core kernels round a probability
+# relative to the largest score seen so far, which in a decode step (cached keys, then the new
+# one) is not the largest of all, and only the loose bound holds there.
+ALIKE_TOL = 1e-5
+ROUNDED_TOL = 1e-2
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C", "D", "G", "H"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "G", "H"])
 def test_bfloat16_against_an_oracle_that_rounds_where_the_engine_does(models, name):
     path, cfg, weights = models[name]
     engine = _engine(path, "bfloat16")
+    plain_kernel = cfg["head_dim"] not in (32, 64, 96, 128, 192, 256)
+
+    def oracle(p):
+        return plain.forward(cfg, weights, p, rounded=plain.round_bfloat16,
+                             rounded_probs=(lambda t: t) if plain_kernel else None)
+    short = [helpers.random_tokens(1 + i % 4, cfg["vocab_size"], 400 + i) for i in range(12)]
+    whole = [helpers.per_position(helpers.run_whole(engine, p), oracle(p)) for p in short]
+    assert max(whole) < ROUNDED_TOL
+    assert sum(e < ALIKE_TOL for e in whole) >= 8, f"whole prompts: {whole}"
+    if plain_kernel:
+        tails = [helpers.per_position(helpers.run_tail_by_one(engine, p, 3), oracle(p)) for p in short]
+        assert max(tails) < ROUNDED_TOL and sum(e < ALIKE_TOL for e in tails) >= 8, f"token by token: {tails}"
     prompts = [helpers.random_tokens(n, cfg["vocab_size"], 300 + i) for i, n in enumerate(LENGTHS[name])]
-    refs = [plain.forward(cfg, weights, p, rounded=plain.round_bfloat16) for p in prompts]
+    refs = [oracle(p) for p in prompts]
     for p, ref in zip(prompts, refs):
         assert helpers.per_position(helpers.run_whole(engine, p), ref) < ROUNDED_TOL, f"whole, length {len(p)}"
         assert helpers.per_position(helpers.run_tail_by_one(engine, p, 32), ref) < ROUNDED_TOL, f"tail, length {len(p)}"

@@ -185,30 +185,32 @@ def test_prompts_far_longer_than_the_window_through_the_entry_point(models, dtyp
     long_prompt = helpers.random_tokens(1000, cfg["vocab_size"], 91)
     short_prompt = helpers.random_tokens(300, cfg["vocab_size"], 92)
     model = Model.load(path, LoadOptions(dtype=dtype, ctx=1100, max_batch=2))
-    windowed = [g for g in model.engine.cache.kv_groups if g.window is not None][0]
-    full = [g for g in model.engine.cache.kv_groups if g.window is None][0]
-    assert windowed.n_pages < full.n_pages
     got = model.generate([long_prompt, short_prompt], max_new_tokens=6)
-    want = [plain.greedy(cfg, w, p, 6) for p in (long_prompt, short_prompt)]
-    for g, wt, p in zip(got, want, (long_prompt, short_prompt)):
-        if dtype == "float32":
-            assert g.tokens == wt
-        elif g.tokens != wt:
-            k = next(i for i in range(6) if g.tokens[i] != wt[i])
-            assert near_tie(cfg, w, p, wt, k)
+    refs = {}
+    for g, p in zip(got, (long_prompt, short_prompt)):
+        # one pass of the plain implementation over prompt and answer: every generated token must be
+        # the best continuation of what stands before it (in bfloat16: or within a near tie of it)
+        assert len(g.tokens) == 6 and g.finish_reason == "length"
+        ref = refs[len(p)] = plain.forward(cfg, w, list(p) + g.tokens)
+        for k, tok in enumerate(g.tokens):
+            row = ref[len(p) - 1 + k]
+            best = int(torch.argmax(row))
+            if tok != best:
+                top = torch.topk(row, 2).values
+                assert dtype == "bfloat16" and float((top[0] - row[tok]) / top[0].abs()) < 1e-2, f"token {k}: {tok} for {best}"
     model.engine.cache.check()
     assert not model.engine.cache.lengths
     # logits, with pieces far smaller than the prompt: the windowed group is then a handful of pages
     engine = Engine(load_model(path, dtype=dtype, device="cuda:0"), max_tokens=2 * 1100, max_seqs=2, max_step_tokens=96)
     windowed = [g for g in engine.cache.kv_groups if g.window is not None][0]
     assert windowed.n_pages == 2 * 4 + 2
-    ref = plain.forward(cfg, w, long_prompt)
+    ref = refs[1000]
     a, b = engine.new_sequence(), engine.new_sequence()
     places = [0, 69, 70, 71, 500, 998, 999]
     logits = engine.step([StepEntry(a, long_prompt[:999], places[:-1]), StepEntry(b, short_prompt[:10], [])]).cpu()
     assert helpers.rel_to_max(logits, ref[places[:-1]]) < tol
     logits = engine.step([StepEntry(a, [long_prompt[999]], [0]), StepEntry(b, [short_prompt[10]], [])]).cpu()
-    assert helpers.rel_to_max(logits, ref[999:]) < tol
+    assert helpers.rel_to_max(logits, ref[999:1000]) < tol
     engine.release(a)
     engine.release(b)
     engine.cache.check()
@@ -236,7 +238,7 @@ def test_generation_stops_at_the_models_end_of_sequence_id(models, tmp_path):
     in_generation_config = str(tmp_path / "generation_config")
     shutil.copytree(path, in_generation_config)
     with open(f"{in_generation_config}/generation_config.json", "w") as f:
-        json.dump({"eos_token_id": [eos, free[6]]}, f)
+        json.dump({"eos_token_id": [eos, next(t for t in range(cfg["vocab_size"]) if t not in free)]}, f)
     model = _load(in_generation_config, "float32", ctx=64, max_batch=1)
     assert model.generate([prompt], max_new_tokens=8)[0].tokens == cut
     assert _load(path, "float32", ctx=64, max_batch=1).generate([prompt], max_new_tokens=8)[0].tokens == free
