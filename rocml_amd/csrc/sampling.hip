@@ -4,6 +4,8 @@
 // keep the top k, softmax, keep the smallest set of most probable tokens whose mass reaches
 // top_p, draw with the caller's uniform number.
 #include "common.h"
+#include "sampling.h"
+#include <mutex>
 
 ROCML_LAST_ERROR_FN(sampling)
 
@@ -770,5 +772,49 @@ ROCML_EXPORT int rocml_argmax(const float* logits, int batch, int vocab, int* ou
         argmax_kernel<<<batch, SB, 0, stream>>>(logits, vocab, out);
     }
     ROCML_CHECK_LAUNCH("argmax");
+    return 0;
+}
+
+// ---- the same without a workspace and without allocating ------------------------------------
+// The partial maxima of rocml_argmax's first stage, in memory of the library itself.  In host
+// code the array's name is not a device address; the address on each GPU is asked for once, with
+// that GPU current, and only that pointer is ever handed to a kernel.
+static __device__ __align__(256) uint32_t g_argmax_static_scratch[2 * ROCML_ARGMAX_STATIC_MAX_ROWS * ARGMAX_CHUNKS];
+
+constexpr int STATIC_MAX_DEVICES = 64;
+static void* g_argmax_static_ptr[STATIC_MAX_DEVICES] = {};
+static std::mutex g_argmax_static_lock;
+
+static int argmax_static_scratch(void** ptr) {
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) return rocml_fail("argmax_static: no current device: %s", hipGetErrorString(e));
+    if (device < 0 || device >= STATIC_MAX_DEVICES)
+        return rocml_fail("argmax_static: device %d is beyond the %d this library keeps an address for", device, STATIC_MAX_DEVICES);
+    std::lock_guard<std::mutex> hold(g_argmax_static_lock);
+    if (!g_argmax_static_ptr[device]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_argmax_static_scratch));
+        if (e != hipSuccess || !p)
+            return rocml_fail("argmax_static: cannot find the scratch array on device %d: %s", device, hipGetErrorString(e));
+        g_argmax_static_ptr[device] = p;
+    }
+    *ptr = g_argmax_static_ptr[device];
+    return 0;
+}
+
+ROCML_EXPORT int rocml_argmax_static(const float* logits, int batch, int vocab, int* out, hipStream_t stream) {
+    ROCML_REQUIRE(batch >= 0 && vocab > 0, "argmax_static: bad sizes B=%d V=%d", batch, vocab);
+    ROCML_REQUIRE(batch <= ROCML_ARGMAX_STATIC_MAX_ROWS, "argmax_static: %d rows exceed the %d the library's scratch array holds",
+                  batch, ROCML_ARGMAX_STATIC_MAX_ROWS);
+    ROCML_REQUIRE(logits && out, "argmax_static: null pointer");
+    if (batch == 0) return 0;
+    void* work = nullptr;
+    if (argmax_static_scratch(&work)) return 1;
+    float* part_val = (float*)work;
+    int* part_idx = (int*)work + (size_t)batch * ARGMAX_CHUNKS;
+    argmax_partial_kernel<<<dim3(ARGMAX_CHUNKS, batch), SB, 0, stream>>>(logits, vocab, part_val, part_idx);
+    argmax_final_kernel<<<batch, 64, 0, stream>>>(part_val, part_idx, out);
+    ROCML_CHECK_LAUNCH("argmax_static");
     return 0;
 }
