@@ -178,6 +178,7 @@ ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, c
 // already), or its split-K partial sums [qkv_splits][tokens][ld], which are added in split
 // order.  q_gain/k_gain null: no norm; cos/sin null: no rotation, else [tokens, D/2].
 // token_seq null: token t is the one token of the step's sequence t (row t of the block table).
+// row_ssq (may be null): the projection's operand lacked its norm's scale (see DecodeProj).
 ROCML_EXPORT int rocml_attention_decode_fused(const float* qkv, int ld, int qkv_splits, long long qkv_split_stride,
                                               const float* q_gain, const float* k_gain, float eps,
                                               const float* cos_t, const float* sin_t, int write_kv, void* out,
@@ -185,7 +186,8 @@ ROCML_EXPORT int rocml_attention_decode_fused(const float* qkv, int ld, int qkv_
                                               const int* token_seq, const int* token_pos, int n_tokens, int hq,
                                               int hkv, int d, int page_size, float scale, int window,
                                               int max_len, int n_splits, void* workspace,
-                                              long long workspace_bytes, hipStream_t stream) {
+                                              long long workspace_bytes, const float* row_ssq, int row_parts,
+                                              float row_eps, int row_width, hipStream_t stream) {
     ROCML_REQUIRE(n_tokens >= 0 && hq > 0 && hkv > 0 && bt_width > 0 && qkv_splits >= 1,
                   "fused decode attention: bad sizes T=%d Hq=%d Hkv=%d width=%d splits=%d", n_tokens, hq, hkv,
                   bt_width, qkv_splits);
@@ -203,7 +205,10 @@ ROCML_EXPORT int rocml_attention_decode_fused(const float* qkv, int ld, int qkv_
     ROCML_REQUIRE((q_gain == nullptr) == (k_gain == nullptr) && (cos_t == nullptr) == (sin_t == nullptr),
                   "fused decode attention: gains and rotation tables come in pairs");
     if (n_tokens == 0) return 0;
-    DecodeProj pj{qkv, ld, qkv_splits, qkv_split_stride, q_gain, k_gain, eps, cos_t, sin_t, write_kv};
+    ROCML_REQUIRE(!row_ssq || (row_parts > 0 && row_eps > 0.f && row_width > 0),
+                  "fused decode attention: a row scale needs parts, eps and the norm's width");
+    DecodeProj pj{qkv, ld, qkv_splits, qkv_split_stride, q_gain, k_gain, eps, cos_t, sin_t, write_kv,
+                  row_ssq, row_parts, row_eps, row_ssq ? 1.0f / (float)row_width : 0.f};
     AttnArgs a{nullptr, (bf16_t*)out, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table, bt_width,
                token_seq, token_pos, nullptr, 0, n_tokens, 0, max_len, hq, hkv, scale, window, workspace,
                workspace_bytes, n_splits, &pj};

@@ -44,10 +44,14 @@ __device__ __forceinline__ float sum_across_halves(float v) {
 // output of the q/k/v projection in 32-bit (or its split-K partial sums, [splits][tokens][ld]),
 // the gains of the per-head norm (null: no norm) and the rotation tables (null: no rotation;
 // else the whole head is rotated, pairs (e, e + D/2)).
+// row_ssq (null: none): the projection's operand was bfloat16(x * gain) of a norm whose scale is
+// still to come; row_ssq[token][row_parts] are sums of squares of x, and every sum of the
+// projection is multiplied by 1 / sqrt(sum of the token's parts * row_inv_width + row_eps) first.
 struct DecodeProj {
     const float* qkv; int ld; int n_splits; long long split_stride;
     const float* q_gain; const float* k_gain; float eps;
     const float* cos_t; const float* sin_t; int write_kv;
+    const float* row_ssq; int row_parts; float row_eps; float row_inv_width;
 };
 
 // grid (n_splits, Hkv, tokens), 4 waves; the block's pages are cut into 32-key pieces that the
@@ -151,6 +155,20 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         owner = pj.write_kv && (last_lpage - first_page) % n_splits == split;
         int n_rows = group + (owner ? 2 : 0);       // q heads, then key, then value
         const float* tok = pj.qkv + (size_t)t * pj.ld;
+        float row_scale = 1.0f;
+        if (pj.row_ssq) {           // (every wave forms the same number in the same order)
+            float ss = 0.f;
+            const float* row = pj.row_ssq + (size_t)t * pj.row_parts;
+            if ((pj.row_parts & 3) == 0) {
+                for (int c = lane; c < pj.row_parts / 4; c += 64) {
+                    float4 v = ((const float4*)row)[c];
+                    ss += (v.x + v.y) + (v.z + v.w);
+                }
+            } else {
+                for (int p = lane; p < pj.row_parts; p += 64) ss += row[p];
+            }
+            row_scale = 1.0f / sqrtf(wave_sum(ss) * pj.row_inv_width + pj.row_eps);
+        }
         for (int base = 0; base < n_rows; base += 2 * (AM_THREADS / 64)) {
             int r[2];
             const float* src[2];
@@ -177,7 +195,7 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                     for (int sp = 1; sp < 4; ++sp)
                         if (sp < pj.n_splits) a += raw[i][j][sp];
                     for (int sp = 4; sp < pj.n_splits; ++sp) a += src[i][j * 64 + sp * pj.split_stride];
-                    val[i][j] = a;
+                    val[i][j] = a * row_scale;
                 }
                 const float* gain = r[i] < group ? pj.q_gain : (r[i] == group ? pj.k_gain : nullptr);
                 if (gain) {

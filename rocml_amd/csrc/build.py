@@ -68,11 +68,23 @@ def build_dir() -> str:
 
 
 def source_hash(family: str) -> str:
-    """Hash of what a family's library is made from: its source, every header of the folder
-    (they are few, and any may be included) and the compiler flags."""
+    """Hash of what a family's library is made from: its source, the headers of this folder that
+    it includes (directly or through another of them) and the compiler flags."""
     h = hashlib.sha256(" ".join([ARCH, *FLAGS]).encode())
-    names = [f"{family}.hip"] + sorted(n for n in os.listdir(SRC_DIR) if n.endswith(".h"))
-    for name in names:
+    names, todo = [], [f"{family}.hip"]
+    while todo:
+        name = todo.pop()
+        if name in names:
+            continue
+        names.append(name)
+        with open(os.path.join(SRC_DIR, name), "r", encoding="utf-8") as f:
+            for line in f:
+                line = line.strip()
+                if line.startswith("#include \""):
+                    inc = line.split('"')[1]
+                    if os.path.exists(os.path.join(SRC_DIR, inc)):
+                        todo.append(inc)
+    for name in sorted(names):
         with open(os.path.join(SRC_DIR, name), "rb") as f:
             h.update(name.encode() + b"\0" + f.read() + b"\0")
     return h.hexdigest()

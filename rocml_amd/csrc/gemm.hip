@@ -21,7 +21,7 @@ static int allow_lds(K kernel, int bytes, const char* name) {
     return 0;
 }
 
-struct SplitPlan { int defer; int* deferred; };
+struct SplitPlan { int defer; int* deferred; RowScale rs; };
 
 template <int EPI, typename T>
 static int launch_mfma_tile_as(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m,
@@ -144,21 +144,21 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
                 (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
         else if constexpr (CAN_NARROW)
             gemm_skinny_kernel<MT, EPI, false, 2><<<grid, 128, LDS, stream>>>(
-                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
+                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split, plan.rs);
     } else if (splits == 1) {
         if constexpr (AHEAD)
             gemm_skinny_ahead_kernel<MT, EPI, false, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
                 (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
         else
             gemm_skinny_kernel<MT, EPI, false, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
-                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
+                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split, plan.rs);
     } else {
         if constexpr (AHEAD)
             gemm_skinny_ahead_kernel<MT, EPI, true, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
                 (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, workspace, n, m, n, k, k_per_split);
         else
             gemm_skinny_kernel<MT, EPI, true, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
-                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, workspace, n, m, n, k, k_per_split);
+                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, workspace, n, m, n, k, k_per_split, RowScale{});
         if (plan.defer && ldo == n) {
             // the caller's next kernel adds the partial sums itself
             *plan.deferred = splits;
@@ -191,10 +191,10 @@ static int launch_kpar(const void* x, int ldx, const void* w, int ldw, void* out
     dim3 grid(n_tiles, splits);
     if (splits == 1) {
         gemm_kpar_kernel<EPI, false><<<grid, GK_THREADS, 0, stream>>>(
-            (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
+            (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split, plan.rs);
     } else {
         gemm_kpar_kernel<EPI, true><<<grid, GK_THREADS, 0, stream>>>(
-            (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, workspace, n, m, n, k, k_per_split);
+            (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, workspace, n, m, n, k, k_per_split, RowScale{});
         if (plan.defer && ldo == n) {
             *plan.deferred = splits;
             return 0;
@@ -242,6 +242,47 @@ ROCML_EXPORT int rocml_splitk_reduce(const float* partials, void* out, int out_d
     return 0;
 }
 
+// resid[M, N] += X * W^T for at most 16 rows of bfloat16 operands, whole sums, and the next norm
+// prepared: xg[M, N] = bfloat16(resid * gain) and ssq[M][ceil(N / 16)], the sums of squares of
+// every 16 columns of a row (see gemm_residual_prescale_kernel).
+ROCML_EXPORT int rocml_gemm_residual_prescale(const void* x, int ldx, const void* w, int ldw, float* resid, int ldr,
+                                              const float* gain, void* xg, int ldg, float* ssq, int m, int n, int k,
+                                              int waves, hipStream_t stream) {
+    ROCML_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm_residual_prescale: bad sizes M=%d N=%d K=%d", m, n, k);
+    ROCML_REQUIRE(m <= 16, "gemm_residual_prescale: at most 16 rows, got %d", m);
+    ROCML_REQUIRE(ldx >= k && ldw >= k && ldr >= n && ldg >= n, "gemm_residual_prescale: row strides (%d, %d, %d, %d) too small",
+                  ldx, ldw, ldr, ldg);
+    ROCML_REQUIRE(k % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0,
+                  "gemm_residual_prescale: K and the operands' row strides must be multiples of 8 and the pointers "
+                  "16-byte aligned (K=%d ldx=%d ldw=%d)", k, ldx, ldw);
+    ROCML_REQUIRE((uintptr_t)resid % 16 == 0 && (uintptr_t)gain % 16 == 0 && (uintptr_t)xg % 8 == 0,
+                  "gemm_residual_prescale: the residual stream, the gain and the prepared operand must be aligned");
+    ROCML_REQUIRE(resid && gain && xg && ssq, "gemm_residual_prescale: null pointer");
+    if (m == 0) return 0;
+    int tiles = ceil_div(n, 16);
+    ROCML_REQUIRE(waves == 0 || waves == 4 || waves == 8 || waves == 16, "gemm_residual_prescale: 4, 8 or 16 waves, got %d", waves);
+    // waves: 0 = choose: eight a block when each still gets 512 of K, else four
+    if (waves == 0) waves = k >= 4096 ? 8 : 4;
+#define GRP_LAUNCH(W_)                                                                                          \
+    gemm_residual_prescale_kernel<W_><<<tiles, 64 * W_, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw, resid, \
+                                                                     ldr, gain, (bf16_t*)xg, ldg, ssq, tiles, m, n, k)
+    if (waves == 16) GRP_LAUNCH(16);
+    else if (waves == 8) GRP_LAUNCH(8);
+    else GRP_LAUNCH(4);
+#undef GRP_LAUNCH
+    ROCML_CHECK_LAUNCH("gemm_residual_prescale");
+    return 0;
+}
+
+// Whether rocml_gemm_residual_prescale is the faster way to add this product to the residual
+// stream and norm the result: its blocks own 16 columns and all of K, so the chip must hold them
+// in one round (256 CUs) and K must be short enough for the eight waves of a block (4096: measured
+// 11.6 us against 21.0 for the product cut along K over blocks plus the norm, at 4096 x 4096 and
+// 8 rows; with K of 12288 the two are equal, beyond that the cut product wins).
+ROCML_EXPORT int rocml_gemm_residual_prescale_pays(int m, int n, int k) {
+    return m >= 1 && m <= 16 && ceil_div(n, 16) <= 256 && k <= 4096 && k % 8 == 0;
+}
+
 // algo: 0 = choose, 1 = plain tiled kernel, 2 = MFMA tile kernel, 3 = MFMA few-rows kernel (M <= 64),
 // 4 = MFMA kernel for at most 16 rows, 5 = MFMA tile kernel with 256x256 tiles.
 // accumulate: out += product (out must be 32-bit); this is the residual sum's epilogue.
@@ -251,10 +292,15 @@ ROCML_EXPORT int rocml_splitk_reduce(const float* partials, void* out, int out_d
 //   the workspace and report their number in *deferred_splits (0 if the product is complete);
 //   the caller's next kernel adds them.  Needs a dense out (ldo == N).
 // workspace: device memory for split-K partial sums (may be null: no split).
+// row_ssq (may be null): X is bfloat16(x * gain) of a norm over K values whose scale is still to
+//   come: row_ssq[M][row_parts] are sums of squares of x whose total over a row gives the row's
+//   scale 1 / sqrt(total / K + row_eps), which the gated epilogue applies to its sums.  Only for
+//   the gated epilogue of at most 16 rows on the MFMA path.
 ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, int w_dtype, int ldw,
                             void* out, int out_dtype, int ldo, int m, int n, int k, int accumulate,
                             int algo, int epilogue, int defer, int* deferred_splits, void* workspace,
-                            long long workspace_bytes, hipStream_t stream) {
+                            long long workspace_bytes, const float* row_ssq, int row_parts, float row_eps,
+                            hipStream_t stream) {
     if (deferred_splits) *deferred_splits = 0;
     ROCML_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm: bad sizes M=%d N=%d K=%d", m, n, k);
     bool gated = epilogue == 1;
@@ -280,13 +326,18 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
     ROCML_REQUIRE(out_dtype == ROCML_F32 || out_dtype == ROCML_BF16, "gemm: unknown output type %d", out_dtype);
     int epi = gated ? EPI_SWIGLU : accumulate ? EPI_ACC : (out_dtype == ROCML_BF16 ? EPI_BF16 : EPI_F32);
     bool use_mfma = mfma_ok && algo != ALGO_PLAIN;
+    if (row_ssq)
+        ROCML_REQUIRE(gated && m <= 16 && use_mfma && row_parts > 0 && row_eps > 0.f &&
+                          (algo == ALGO_AUTO || algo == ALGO_MFMA_SKINNY || algo == ALGO_MFMA_KPAR),
+                      "gemm: a row scale goes with the gated epilogue of at most 16 rows on the few-rows MFMA kernels "
+                      "(M=%d parts=%d)", m, row_parts);
     if (use_mfma) {
         // Up to 16 rows the few-rows kernels; up to 64 rows still for the gated product (it cannot
         // cut K in pieces, which is what the tile kernel lives on with so few rows) and, up to 32
         // rows, for every product but the widest (the output projection over the vocabulary).
         bool few_rows = m <= 16 || (m <= 64 && (gated || (m <= 32 && n < 65536)));
         bool skinny = algo == ALGO_MFMA_SKINNY || (algo == ALGO_AUTO && few_rows);
-        SplitPlan plan{defer, deferred_splits};
+        SplitPlan plan{defer, deferred_splits, RowScale{row_ssq, row_parts, row_eps, 1.0f / (float)k}};
         int rc;
 #define BY_EPI(fn, ...)                                              \
         (epi == EPI_F32 ? fn<EPI_F32>(__VA_ARGS__)                   \

@@ -42,6 +42,71 @@ enum GemmEpilogue : int { EPI_F32 = 0, EPI_BF16 = 1, EPI_ACC = 2, EPI_SWIGLU = 3
 
 __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
 
+// The scale of a norm whose product-side half was done by the producer of the residual stream
+// (gemm_residual_prescale_kernel): the operand is bfloat16(x * gain), and the sums of this product
+// still lack the factor 1 / sqrt(sum of x^2 / width + eps) of their row, which is formed here from
+// the sums of squares per 16 columns that the producer left.  ssq null: nothing to scale.
+struct RowScale { const float* ssq; int parts; float eps; float inv_width; };
+
+// The scale of activation row lane%16 (the row an MFMA lane's sums belong to), the same in the
+// four lanes of a row; rows beyond M get 1.  In two steps: row_scale_request (the whole wave works
+// on every row: a lane loads a sixteenth or less of the row's sums, all rows' loads go out
+// together, one trip to memory) and row_scale_finish (the lanes' sums meet by butterfly, in the
+// same order whatever the row).
+__device__ __forceinline__ void row_scale_request(RowScale rs, int lane, int m, float (&part)[16]) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) part[r] = 0.f;
+    if (!rs.ssq) return;
+    // No branch between the loads of different rows (a branch would make every row wait for its own
+    // trip): rows beyond M read the last row again, lanes beyond the row's end read its start, and
+    // what they read is not counted.
+    if ((rs.parts & 3) == 0) {
+        int chunks = rs.parts / 4;
+        const float4* all = (const float4*)rs.ssq;
+        for (int base = 0; base < chunks; base += 64) {
+            bool ok = base + lane < chunks;
+            int c = ok ? base + lane : 0;
+            float4 v[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) v[r] = all[(size_t)min(r, m - 1) * chunks + c];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) part[r] += ok ? (v[r].x + v[r].y) + (v[r].z + v[r].w) : 0.f;
+        }
+    } else {
+        for (int base = 0; base < rs.parts; base += 64) {
+            bool ok = base + lane < rs.parts;
+            int p = ok ? base + lane : 0;
+            float v[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) v[r] = rs.ssq[(size_t)min(r, m - 1) * rs.parts + p];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) part[r] += ok ? v[r] : 0.f;
+        }
+    }
+}
+
+// red: 16 x RS_RED_STRIDE floats of LDS that the calling wave has to itself.  The lanes' sums meet
+// there: every lane leaves its sixteen partial sums, then adds up a quarter of the row lane%16 and
+// two butterfly steps finish it (a butterfly per row would be 96 exchanges instead of 2).
+constexpr int RS_RED_STRIDE = 68;     // 16-byte aligned rows whose banks are staggered
+
+__device__ __forceinline__ float row_scale_finish(RowScale rs, int lane, int m, const float (&part)[16], float* red) {
+    if (!rs.ssq) return 1.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) red[r * RS_RED_STRIDE + lane] = part[r];
+    __builtin_amdgcn_wave_barrier();
+    const float4* mine = (const float4*)(red + (lane & 15) * RS_RED_STRIDE + (lane >> 4) * 16);
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float4 v = mine[j];
+        s += (v.x + v.y) + (v.z + v.w);
+    }
+    s += __shfl_xor(s, 16, 64);
+    s += __shfl_xor(s, 32, 64);
+    return (lane & 15) < m ? 1.0f / sqrtf(s * rs.inv_width + rs.eps) : 1.0f;
+}
+
 template <int EPI>
 __device__ __forceinline__ void epilogue_store(void* out, size_t idx, float v) {
     if (EPI == EPI_F32) ((float*)out)[idx] = v;
@@ -253,7 +318,7 @@ constexpr int GS_ROW = GS_KC / 8 + 1;                 // uint4 per LDS row of ac
 // Accumulator element e of a lane: weight row (lane/16)*4 + e, activation row lane%16.
 template <int MT, int EPI, bool PARTIAL>
 __device__ __forceinline__ void skinny_epilogue(const f32x4_t (&acc)[MT], void* out, int ldo, int m, int n, int n0,
-                                                int lane, int split) {
+                                                int lane, int split, float row_scale = 1.0f) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         int gm = mt * 16 + (lane & 15);
@@ -264,7 +329,8 @@ __device__ __forceinline__ void skinny_epilogue(const f32x4_t (&acc)[MT], void* 
             for (int e = 0; e < 4; e += 2) {
                 int gn = n0 + (lane >> 4) * 4 + e;
                 if (gn + 1 < n)
-                    ((bf16_t*)out)[(size_t)gm * ldo + (gn >> 1)] = f32_to_bf16(silu_mul(acc[mt][e], acc[mt][e + 1]));
+                    ((bf16_t*)out)[(size_t)gm * ldo + (gn >> 1)] =
+                        f32_to_bf16(silu_mul(acc[mt][e] * row_scale, acc[mt][e + 1] * row_scale));
             }
             continue;
         }
@@ -287,7 +353,7 @@ __device__ __forceinline__ void skinny_epilogue(const f32x4_t (&acc)[MT], void* 
 template <int MT, int EPI, bool PARTIAL, int WAVES = 4>
 __global__ void __launch_bounds__(64 * WAVES)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw,
-                   void* __restrict__ out, int ldo, int m, int n, int k, int k_per_split) {
+                   void* __restrict__ out, int ldo, int m, int n, int k, int k_per_split, RowScale rs) {
     extern __shared__ u32x4_t gs_smem[];              // [2][MT*16][GS_ROW]
     constexpr int ROWS = MT * 16;
     constexpr int THREADS = 64 * WAVES;
@@ -340,6 +406,19 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restri
 
     GS_LOAD_W(0, wcur)
     GS_LOAD_X(0)
+    // The rows' scales, if the operand lacks them (only the gated epilogue of at most 16 rows
+    // applies them): the block's first wave forms them while the first weights are on their way
+    // and leaves them in LDS for the epilogue.  (Held in registers through the loop they cost the
+    // kernel a wave per SIMD; asked for in the epilogue, a trip to memory at the kernel's end.)
+    constexpr bool SCALES = MT == 1 && EPI == EPI_SWIGLU && !PARTIAL;
+    __shared__ float gs_scale[16];
+    __shared__ __attribute__((aligned(16))) float gs_red[SCALES ? 16 * RS_RED_STRIDE : 4];
+    if (SCALES && wave == 0) {
+        float scale_part[16];
+        row_scale_request(rs, lane, m, scale_part);
+        float mine = row_scale_finish(rs, lane, m, scale_part, gs_red);
+        if (lane < 16) gs_scale[lane] = mine;
+    }
     GS_STORE_X(0, 0)
     __syncthreads();
     for (int c = 0; c < n_chunks; ++c) {
@@ -370,7 +449,8 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restri
 #undef GS_LOAD_W
 #undef GS_LOAD_X
 #undef GS_STORE_X
-    skinny_epilogue<MT, EPI, PARTIAL>(acc, out, ldo, m, n, n0, lane, blockIdx.y);
+    float row_scale = SCALES ? gs_scale[lane & 15] : 1.0f;
+    skinny_epilogue<MT, EPI, PARTIAL>(acc, out, ldo, m, n, n0, lane, blockIdx.y, row_scale);
 }
 
 // The same product for 17 to 64 rows.  With more rows a step costs more (four products and four
@@ -525,7 +605,7 @@ constexpr int GK_KC = 256, GK_THREADS = 256;
 template <int EPI, bool PARTIAL>
 __global__ void __launch_bounds__(GK_THREADS)
 gemm_kpar_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw,
-                 void* __restrict__ out, int ldo, int m, int n, int k, int k_per_split) {
+                 void* __restrict__ out, int ldo, int m, int n, int k, int k_per_split, RowScale rs) {
     __shared__ float red[4][64][4];
     int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int g = lane >> 4, col = lane & 15;
@@ -549,6 +629,17 @@ gemm_kpar_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
         xd_[j] = *(const u32x4_t*)(in_ ? xp + (kb_) + j * 32 : xsafe);        \
     }
     if (ks < ke) GK_LOAD(ks, wc, xc)
+    // (the rows' scales for the gated epilogue: formed by the last wave while its first loads are
+    // on their way, handed to the first wave through LDS)
+    constexpr bool SCALES = EPI == EPI_SWIGLU && !PARTIAL;
+    __shared__ float gk_scale[16];
+    __shared__ __attribute__((aligned(16))) float gk_red[SCALES ? 16 * RS_RED_STRIDE : 4];
+    if (SCALES && wave == 3) {
+        float scale_part[16];
+        row_scale_request(rs, lane, m, scale_part);
+        float mine = row_scale_finish(rs, lane, m, scale_part, gk_red);
+        if (lane < 16) gk_scale[lane] = mine;
+    }
     for (int kb = ks; kb < ke; kb += GK_KC) {
         bool more = kb + GK_KC < ke;
         if (more) GK_LOAD(kb + GK_KC, wn, xn)
@@ -570,7 +661,9 @@ gemm_kpar_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
 #pragma unroll
     for (int e = 0; e < 4; ++e) red[wave][lane][e] = acc[e];
     __syncthreads();
-    if (wave != 0 || !xok) return;
+    if (wave != 0) return;
+    float row_scale = SCALES ? gk_scale[lane & 15] : 1.0f;
+    if (!xok) return;
     float sum[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) sum[e] = ((red[0][lane][e] + red[1][lane][e]) + red[2][lane][e]) + red[3][lane][e];
@@ -580,7 +673,8 @@ gemm_kpar_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
 #pragma unroll
         for (int e = 0; e < 4; e += 2)
             if (gn0 + e + 1 < n)
-                ((bf16_t*)out)[(size_t)col * ldo + ((gn0 + e) >> 1)] = f32_to_bf16(silu_mul(sum[e], sum[e + 1]));
+                ((bf16_t*)out)[(size_t)col * ldo + ((gn0 + e) >> 1)] =
+                    f32_to_bf16(silu_mul(sum[e] * row_scale, sum[e + 1] * row_scale));
         return;
     }
 #pragma unroll
@@ -590,6 +684,102 @@ gemm_kpar_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
         if (PARTIAL) ((float*)out)[((size_t)split * m + col) * n + gn] = sum[e];
         else epilogue_store<EPI>(out, (size_t)col * ldo + gn, sum[e]);
     }
+}
+
+// ---- at most 16 rows: the residual sum, and the next norm prepared ------------------------------
+// resid[M, N] += X[M, K] * W[N, K]^T with whole sums (a block owns 16 weight rows and all of K; its
+// waves split K and meet once in LDS, in wave order), and in the same pass what the norm that
+// reads the residual stream next would otherwise need a kernel of its own for: xg = bfloat16(resid *
+// gain), the operand of the next product up to the row's scale, and ssq[row][tile], the sum of
+// squares of the block's 16 columns of the row.  Whoever consumes the next product's sums
+// multiplies them by 1 / sqrt(sum of ssq[row] / N + eps): the norm's scale is one number per row
+// and commutes with the product.  A decode step of a few sequences is priced by the kernels that
+// follow one another, not by bytes; this takes two norms out of every layer.
+template <int WAVES>
+__global__ void __launch_bounds__(64 * WAVES)
+gemm_residual_prescale_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw,
+                              float* resid, int ldr, const float* __restrict__ gain, bf16_t* __restrict__ xg, int ldg,
+                              float* __restrict__ ssq, int tiles, int m, int n, int k) {
+    __shared__ float red[WAVES][64][4];
+    int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int g = lane >> 4, col = lane & 15;
+    int tile = blockIdx.x;
+    int share = (((k + WAVES - 1) / WAVES) + 31) / 32 * 32;
+    int ks = min(k, wave * share), ke = min(k, ks + share);
+    const bf16_t* wsafe = w + (size_t)min(tile * 16 + col, n - 1) * ldw;
+    const bf16_t* xsafe = x + (size_t)min(col, m - 1) * ldx;
+    const bf16_t* wp = wsafe + g * 8;
+    const bf16_t* xp = xsafe + g * 8;
+    u32x4_t wc[8], xc[8], wn[8], xn[8];
+    f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    bool xrow = col < m;        // lanes of rows beyond M load no activations (their sums are not stored)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) xc[j] = xn[j] = u32x4_t{0u, 0u, 0u, 0u};
+    // (no select behind a load: clamped addresses; a piece beyond the wave's K range is zeroed on
+    // the activation side just before it is multiplied)
+#define GR_LOAD(kb_, wd_, xd_)                                                \
+    _Pragma("unroll") for (int j = 0; j < 8; ++j) {                           \
+        bool in_ = (kb_) + j * 32 + g * 8 < ke;                               \
+        wd_[j] = *(const u32x4_t*)(in_ ? wp + (kb_) + j * 32 : wsafe);        \
+        if (xrow) xd_[j] = *(const u32x4_t*)(in_ ? xp + (kb_) + j * 32 : xsafe); \
+    }
+    if (ks < ke) GR_LOAD(ks, wc, xc)
+    for (int kb = ks; kb < ke; kb += GK_KC) {
+        bool more = kb + GK_KC < ke;
+        if (more) GR_LOAD(kb + GK_KC, wn, xn)
+        const u32x4_t zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            u32x4_t xv = kb + j * 32 + g * 8 < ke ? xc[j] : zero;
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag4(wc[j]), as_frag4(xv), acc, 0, 0, 0);
+        }
+        if (more) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                wc[j] = wn[j];
+                xc[j] = xn[j];
+            }
+        }
+    }
+#undef GR_LOAD
+#pragma unroll
+    for (int e = 0; e < 4; ++e) red[wave][lane][e] = acc[e];
+    __syncthreads();
+    if (wave != 0) return;
+    // element e of a lane: weight row (output column) 16 tile + 4g + e, activation row lane%16
+    float v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        float sum = red[0][lane][e];
+#pragma unroll
+        for (int wv = 1; wv < WAVES; ++wv) sum += red[wv][lane][e];
+        v[e] = sum;
+    }
+    int n0 = tile * 16 + g * 4;
+    bool row_ok = col < m;
+    float ss = 0.f;
+    if (row_ok && n0 + 3 < n && (ldr & 3) == 0 && (ldg & 3) == 0) {
+        float4* rp = (float4*)(resid + (size_t)col * ldr + n0);
+        float4 r = *rp;
+        float4 gn = *(const float4*)(gain + n0);
+        r.x += v[0]; r.y += v[1]; r.z += v[2]; r.w += v[3];
+        *rp = r;
+        *(uint2*)(xg + (size_t)col * ldg + n0) = make_uint2(f32x2_to_bf16x2(r.x * gn.x, r.y * gn.y),
+                                                             f32x2_to_bf16x2(r.z * gn.z, r.w * gn.w));
+        ss = fmaf(r.x, r.x, fmaf(r.y, r.y, fmaf(r.z, r.z, r.w * r.w)));
+    } else if (row_ok) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (n0 + e >= n) continue;
+            float r = resid[(size_t)col * ldr + n0 + e] + v[e];
+            resid[(size_t)col * ldr + n0 + e] = r;
+            xg[(size_t)col * ldg + n0 + e] = f32_to_bf16(r * gain[n0 + e]);
+            ss = fmaf(r, r, ss);
+        }
+    }
+    ss += __shfl_xor(ss, 16, 64);
+    ss += __shfl_xor(ss, 32, 64);
+    if (row_ok && g == 0) ssq[(size_t)col * tiles + tile] = ss;
 }
 
 // out[m][n] (+)= sum over splits, in split order.

@@ -42,6 +42,7 @@ class StepContext:
     memo: Dict = field(default_factory=dict)
     block_tables: Dict = field(default_factory=dict)   # cache group name -> [B, width] int32
     want_rows: Optional[torch.Tensor] = None           # token rows whose logits are wanted
+    row_scale: Optional[object] = None                 # set around a part's forward: its input lacks this scale
 
     @property
     def is_decode(self) -> bool:
@@ -51,19 +52,14 @@ class StepContext:
 def pack_step(slots: Sequence[int], starts: Sequence[int], tokens: Sequence[Sequence[int]]):
     """Host arrays of a packed step: ids, sequence index and position per token, offsets,
     final lengths."""
-    counts = [len(t) for t in tokens]
-    total = sum(counts)
-    ids = np.empty(total, dtype=np.int32)
-    seq = np.empty(total, dtype=np.int32)
-    pos = np.empty(total, dtype=np.int32)
+    counts = np.asarray([len(t) for t in tokens], dtype=np.int32)
+    total = int(counts.sum())
     cu = np.zeros(len(tokens) + 1, dtype=np.int32)
-    at = 0
-    for b, (start, toks) in enumerate(zip(starts, tokens)):
-        n = len(toks)
-        ids[at:at + n] = toks
-        seq[at:at + n] = b
-        pos[at:at + n] = np.arange(start, start + n, dtype=np.int32)
-        at += n
-        cu[b + 1] = at
-    lens = np.asarray([s + c for s, c in zip(starts, counts)], dtype=np.int32)
+    np.cumsum(counts, out=cu[1:])
+    ids = np.fromiter((t for toks in tokens for t in toks), dtype=np.int32, count=total)
+    seq = np.repeat(np.arange(len(tokens), dtype=np.int32), counts)
+    first = np.asarray(starts, dtype=np.int32)
+    # position of a token = its sequence's start + its place among the sequence's new tokens
+    pos = np.arange(total, dtype=np.int32) - np.repeat(cu[:-1], counts) + np.repeat(first, counts)
+    lens = first + counts
     return ids, seq, pos, cu, lens, np.asarray(slots, dtype=np.int32)

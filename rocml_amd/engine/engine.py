@@ -82,35 +82,40 @@ class Engine:
         if len(set(slots)) != len(slots):
             raise RocmlError("a sequence appears twice in one step")
         starts, new_lens = [], []
-        for e in entries:
+        counts = [len(e.tokens) for e in entries]
+        if min(counts) == 0:
+            raise RocmlError("a step entry needs at least one token")
+        # one look at all ids together; the entry at fault is searched for only when there is one
+        flat = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=sum(counts))
+        if int(flat.min()) < 0 or int(flat.max()) >= spec.vocab:
+            bad = int(flat[(flat < 0) | (flat >= spec.vocab)][0])
+            raise RocmlError(f"token id {bad} is outside the vocabulary of {spec.vocab}")
+        for e, n in zip(entries, counts):
             if not self.cache.slots.is_live(e.slot):
                 raise RocmlError(f"slot {e.slot} is not a live sequence")
-            if len(e.tokens) == 0:
-                raise RocmlError("a step entry needs at least one token")
-            ids = np.asarray(e.tokens, dtype=np.int64)
-            if int(ids.min()) < 0 or int(ids.max()) >= spec.vocab:
-                bad = int(ids[(ids < 0) | (ids >= spec.vocab)][0])
-                raise RocmlError(f"token id {bad} is outside the vocabulary of {spec.vocab}")
             for w in e.want:
-                if not 0 <= int(w) < len(e.tokens):
-                    raise RocmlError(f"wanted place {w} is outside the entry's {len(e.tokens)} tokens")
+                if not 0 <= int(w) < n:
+                    raise RocmlError(f"wanted place {w} is outside the entry's {n} tokens")
             start = self.cache.length(e.slot)
-            if start + len(e.tokens) > spec.max_positions:
+            if start + n > spec.max_positions:
                 raise ContextOverflowError(
-                    f"sequence would reach {start + len(e.tokens)} positions; the model has "
+                    f"sequence would reach {start + n} positions; the model has "
                     f"{spec.max_positions}")
             starts.append(start)
-            new_lens.append(start + len(e.tokens))
+            new_lens.append(start + n)
         # The step as pieces of at most max_step_tokens tokens (a sequence may straddle pieces).
         # Pages are reserved piece by piece, and a piece is committed before the next runs, so a
         # group with a window gives pages back while a long prompt passes through it; the whole
         # plan is checked against the free pages first, so a step runs entirely or not at all.
-        pieces = self.plan_pieces([len(e.tokens) for e in entries])
-        short = self.cache.fits([[(entries[i].slot, starts[i] + hi) for i, _, hi in piece] for piece in pieces])
-        if short is not None:
-            raise CacheFullError(short)
+        total = sum(counts)
         n_want_total = sum(len(e.want) for e in entries)
-        if len(pieces) == 1:
+        pieces = None
+        if total > self.max_step_tokens:
+            pieces = self.plan_pieces(counts)
+            short = self.cache.fits([[(entries[i].slot, starts[i] + hi) for i, _, hi in piece] for piece in pieces])
+            if short is not None:
+                raise CacheFullError(short)
+        if pieces is None:             # one piece: its reservation is all or nothing by itself
             self.cache.reserve(slots, new_lens)
             logits = self._run_piece(slots, starts, [list(e.tokens) for e in entries],
                                      [list(e.want) for e in entries])

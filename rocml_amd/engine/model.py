@@ -164,7 +164,15 @@ class DecoderModel:
             block = self.blocks[entry.layer]
             if not getattr(block, "takes_pending", False):
                 ws.flush_pending()
-            block.forward(step, x, view, owner == i)
+            # the block that runs next may let this block's last product prepare its first norm
+            following = self.blocks[s.schedule[i + 1].layer] if i + 1 < len(s.schedule) else None
+            hint = None
+            if getattr(block, "takes_next_norm", False) and hasattr(following, "entry_hint"):
+                hint = following.entry_hint(step)
+            if hint is not None:
+                block.forward(step, x, view, owner == i, next_norm=hint)
+            else:
+                block.forward(step, x, view, owner == i)
         if n_want == 0:
             ws.drop_pending()
             return None

@@ -36,14 +36,16 @@ _SIGNATURES = {
         "rocml_add_into": [_P, _P, _I, _LL, _P],
     },
     "gemm": {
-        "rocml_gemm": [_P, _I, _I, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _LL, _P],
+        "rocml_gemm": [_P, _I, _I, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _LL, _P, _I, _F, _P],
         "rocml_splitk_reduce": [_P, _P, _I, _I, _I, _I, _I, _I, _P],
+        "rocml_gemm_residual_prescale_pays": [_I, _I, _I],
+        "rocml_gemm_residual_prescale": [_P, _I, _P, _I, _P, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P],
     },
     "attention": {
         "rocml_attention": [_P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I,
                             _P, _I, _I, _P, _I, _I, _P, _LL, _P],
         "rocml_attention_decode_fused": [_P, _I, _I, _LL, _P, _P, _F, _P, _P, _I, _P, _P, _P, _P, _I, _P, _P,
-                                         _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _LL, _P],
+                                         _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _LL, _P, _I, _F, _I, _P],
     },
     "sampling": {
         "rocml_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _P],
@@ -243,17 +245,33 @@ def add_into(x: torch.Tensor, y: torch.Tensor) -> None:
 
 # ---- matrix product ------------------------------------------------------------------
 GEMM_AUTO, GEMM_PLAIN = 0, 1
+ROW_SCALE_MAX_ROWS = 16     # most rows of a product whose consumer applies a row scale
+
+
+class RowScale:
+    """What is left of a norm whose operand ``bfloat16(x * gain)`` was prepared by the product that
+    completed ``x`` (``gemm_residual_prescale``): ``ssq [rows, parts]`` float32 sums of squares
+    whose total over a row, divided by ``width`` and with ``eps`` added, is the square of what the
+    row still has to be divided by.  The consumer of the next product applies it to its sums."""
+
+    def __init__(self, ssq: torch.Tensor, eps: float, width: int):
+        _dev(ssq)
+        _want(ssq, torch.float32, "sums of squares")
+        if ssq.dim() != 2:
+            raise KernelError("sums of squares must be [rows, parts]")
+        self.ssq, self.eps, self.width = ssq, float(eps), int(width)
 
 
 def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
          algo: int = GEMM_AUTO, workspace: Optional[torch.Tensor] = None, epilogue: Optional[str] = None,
-         defer: bool = False) -> int:
+         defer: bool = False, row_scale: Optional["RowScale"] = None) -> int:
     """``out (+)= x @ w.T`` for ``x [M, K]``, ``w [N, K]``, ``out [M, N]`` (rows may be
     strided views with unit inner stride).  ``epilogue="swiglu"``: ``w``'s rows are (gate, up)
     pairs and ``out`` is ``[M, N/2] = silu(gate) * up``.  With ``defer`` a product that was
     split along K leaves its partial sums ``[splits, M, N]`` at the start of ``workspace`` and
     returns their number for the caller's next kernel to add; it returns 0 when ``out`` is
-    complete."""
+    complete.  ``row_scale``: ``x`` lacks its norm's scale (see ``RowScale``), which the gated
+    epilogue applies; at most ``ROW_SCALE_MAX_ROWS`` rows."""
     for t in (x, w, out):
         if not t.is_cuda:
             raise KernelError("kernel arguments must be GPU tensors; this library has no CPU path")
@@ -268,12 +286,62 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         raise KernelError(f"matrix product shapes do not fit: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
     ws_ptr, ws_bytes = (None, 0) if workspace is None else (workspace.data_ptr(), workspace.numel() * workspace.element_size())
     deferred = ctypes.c_int(0)
+    ssq_ptr, parts, eps = None, 0, 0.0
+    if row_scale is not None:
+        if epilogue != "swiglu" or m > ROW_SCALE_MAX_ROWS or row_scale.width != k or row_scale.ssq.shape[0] < m:
+            raise KernelError("a row scale goes with the gated epilogue of at most 16 rows whose K is the norm's width")
+        ssq_ptr, parts, eps = row_scale.ssq.data_ptr(), row_scale.ssq.shape[1], row_scale.eps
     _check("gemm", library("gemm").rocml_gemm(
         _ptr(x), _code(x), x.stride(0) if m > 1 else max(x.stride(0), k), _ptr(w), _code(w), w.stride(0),
         _ptr(out), _code(out), out.stride(0) if m > 1 else max(out.stride(0), cols), m, n, k,
         1 if accumulate else 0, algo, 1 if epilogue else 0, 1 if defer else 0, ctypes.byref(deferred), ws_ptr,
-        ws_bytes, _stream()))
+        ws_bytes, ssq_ptr, parts, eps, _stream()))
     return deferred.value
+
+
+PRESCALE_MAX_ROWS = 16      # most rows gemm_residual_prescale takes
+PRESCALE_TILE = 16          # columns whose squares one entry of its sums of squares covers
+
+
+def gemm_residual_prescale_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether ``gemm_residual_prescale`` takes this product."""
+    return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and 1 <= x.shape[0] <= PRESCALE_MAX_ROWS
+            and x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0)
+
+
+def gemm_residual_prescale_pays(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether it takes the product and is the faster way (the library's own rule)."""
+    return gemm_residual_prescale_fits(x, w) and \
+        library("gemm").rocml_gemm_residual_prescale_pays(x.shape[0], w.shape[0], x.shape[1]) != 0
+
+
+def gemm_residual_prescale(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, gain: torch.Tensor,
+                           xg: torch.Tensor, ssq: torch.Tensor, waves: int = 0) -> None:
+    """``resid += x @ w.T`` (whole sums, at most 16 rows of bfloat16 operands) and, for the norm
+    with ``gain`` that reads ``resid`` next: ``xg = bfloat16(resid * gain)`` and ``ssq[row][j]`` =
+    the sum of squares of columns ``16 j .. 16 j + 15`` of the row.  The norm's output is
+    ``xg * (1 / sqrt(ssq[row].sum() / N + eps))``; the scale commutes with the next product."""
+    _dev(gain, ssq)
+    for t in (x, w, resid, xg):
+        if not t.is_cuda:
+            raise KernelError("kernel arguments must be GPU tensors; this library has no CPU path")
+        if t.dim() != 2 or t.stride(1) != 1:
+            raise KernelError("matrix product operands must be 2-D with unit inner stride")
+    m, k = x.shape
+    n = w.shape[0]
+    if not gemm_residual_prescale_fits(x, w):
+        raise KernelError(f"gemm_residual_prescale does not take x {tuple(x.shape)} {x.dtype}, w {tuple(w.shape)} {w.dtype}")
+    _want(resid, torch.float32, "residual stream")
+    _want(gain, torch.float32, "norm gain")
+    _want(xg, torch.bfloat16, "prepared operand")
+    _want(ssq, torch.float32, "sums of squares")
+    tiles = (n + PRESCALE_TILE - 1) // PRESCALE_TILE
+    if w.shape[1] != k or resid.shape != (m, n) or xg.shape != (m, n) or gain.numel() != n or ssq.shape != (m, tiles):
+        raise KernelError(f"shapes do not fit: x {tuple(x.shape)}, w {tuple(w.shape)}, residual {tuple(resid.shape)}, "
+                          f"prepared {tuple(xg.shape)}, gain {gain.numel()}, sums {tuple(ssq.shape)} (need {(m, tiles)})")
+    _check("gemm", library("gemm").rocml_gemm_residual_prescale(
+        _ptr(x), max(x.stride(0), k), _ptr(w), w.stride(0), _ptr(resid), max(resid.stride(0), n), _ptr(gain), _ptr(xg),
+        max(xg.stride(0), n), _ptr(ssq), m, n, k, waves, _stream()))
 
 
 def splitk_reduce(partials: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
@@ -333,6 +401,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache
 
 
 FUSED_DECODE_HEAD_DIMS = (64, 128, 192, 256)
+FUSED_DECODE_PAGE = 64
 
 
 def attention_decode_fusable(dtype: torch.dtype, n_heads: int, n_kv_heads: int, head_dim: int, page: int,
@@ -350,12 +419,13 @@ def attention_decode_fused(qkv: torch.Tensor, out: torch.Tensor, k_cache: torch.
                            q_gain: Optional[torch.Tensor], k_gain: Optional[torch.Tensor], eps: float,
                            cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], write_kv: bool = True,
                            window: Optional[int] = None, workspace: Optional[torch.Tensor] = None,
-                           max_len: int = 0, n_splits: int = 0) -> None:
+                           max_len: int = 0, n_splits: int = 0, row_scale: Optional[RowScale] = None) -> None:
     """A decode step's attention straight from the q/k/v projection ``qkv`` (float32
     ``[tokens, ld]``, or its split-K partial sums ``[splits, tokens, ld]``): per-head norm,
     rotation, append of the new key and value to the cache and attention over the cache in one
     launch.  ``token_seq`` None: token ``t`` is the one token of the step's sequence ``t`` (row
-    ``t`` of the block table).  ``workspace`` must not overlap ``qkv``."""
+    ``t`` of the block table).  ``workspace`` must not overlap ``qkv``.  ``row_scale``: the
+    projection's operand lacked its norm's scale, which is applied to the projection's sums here."""
     _dev(qkv, out, k_cache, v_cache, block_table, token_seq, token_pos, q_gain, k_gain, cos, sin)
     _want(qkv, torch.float32, "projection output")
     qkv_splits, split_stride = 1, 0
@@ -391,11 +461,17 @@ def attention_decode_fused(qkv: torch.Tensor, out: torch.Tensor, k_cache: torch.
     if (token_seq is not None and token_seq.numel() != n_tokens) or token_pos.numel() != n_tokens:
         raise KernelError("one sequence index and one position per token are needed")
     ws_ptr, ws_bytes = (None, 0) if workspace is None else (workspace.data_ptr(), workspace.numel() * workspace.element_size())
+    ssq_ptr, parts, row_eps, width = None, 0, 0.0, 0
+    if row_scale is not None:
+        if row_scale.ssq.shape[0] < n_tokens:
+            raise KernelError("the row scale has fewer rows than the step has tokens")
+        ssq_ptr, parts, row_eps, width = row_scale.ssq.data_ptr(), row_scale.ssq.shape[1], row_scale.eps, row_scale.width
     _check("attention", library("attention").rocml_attention_decode_fused(
         _ptr(qkv), ld, qkv_splits, split_stride, _ptr(q_gain), _ptr(k_gain), eps, _ptr(cos), _ptr(sin),
         1 if write_kv else 0, _ptr(out), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
         _ptr(token_seq), _ptr(token_pos), n_tokens, n_heads, n_kv_heads, head_dim, page, scale,
-        0 if window is None else int(window), max_len, n_splits, ws_ptr, ws_bytes, _stream()))
+        0 if window is None else int(window), max_len, n_splits, ws_ptr, ws_bytes, ssq_ptr, parts, row_eps, width,
+        _stream()))
 
 
 # ---- sampling ------------------------------------------------------------------------

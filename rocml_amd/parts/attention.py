@@ -81,6 +81,15 @@ class Attention(Mixer):
         rot = 0 if self.position is None else 2 * n_tokens * (self.position.rot_dim // 2) * 4
         return n_tokens * ((self.q_dim + 2 * self.kv_dim) * 4 + 2 * self.q_dim * size) + rot
 
+    def _fused_decode(self, step) -> bool:
+        rot = None if self.position is None else self.position.rot_dim
+        return step.max_new == 1 and ops.attention_decode_fusable(
+            self.dtype, self.spec.n_heads, self.spec.n_kv_heads, self.spec.head_dim, ops.FUSED_DECODE_PAGE, rot)
+
+    def takes_row_scale(self, step) -> bool:
+        # only the decode kernel that reads the projection's sums itself applies a scale to them
+        return self._fused_decode(step)
+
     def cache_request(self) -> KVCacheRequest:
         return KVCacheRequest(self.spec.n_kv_heads, self.spec.head_dim, self.spec.window)
 
@@ -110,8 +119,7 @@ class Attention(Mixer):
             rot = self.position.rot_dim
         eps = s.qk_norm.eps if s.qk_norm is not None else 1.0
         o = ws.get("attn.o", (n, self.q_dim), self.dtype)
-        if step.max_new == 1 and ops.attention_decode_fusable(cache.k.dtype, s.n_heads, s.n_kv_heads, s.head_dim,
-                                                               cache.k.shape[2], rot if cos is not None else None):
+        if self._fused_decode(step) and cache.k.dtype == self.dtype and cache.k.shape[2] == ops.FUSED_DECODE_PAGE:
             # One token per sequence: norm, rotation, append and attention in one launch, straight
             # from the projection.  The attention's own partial results go behind the projection's.
             used = (splits * n * rows * 4 + 255) // 256 * 256 if splits else 0
@@ -119,8 +127,11 @@ class Attention(Mixer):
             ops.attention_decode_fused(qkv, o, cache.k, cache.v, cache.block_table, None, step.token_pos,
                                        s.n_heads, s.n_kv_heads, s.head_dim, s.scale, self.q_gain, self.k_gain, eps,
                                        cos, sin, write_kv=owns_cache, window=s.window, workspace=scratch[used:],
-                                       max_len=step.max_len, n_splits=self._decode_splits(step, cache))
+                                       max_len=step.max_len, n_splits=self._decode_splits(step, cache),
+                                       row_scale=step.row_scale)
         else:
+            if step.row_scale is not None:
+                raise ConfigError("the attention was handed an input without its norm's scale in a step it cannot scale")
             q = ws.get("attn.q", (n, self.q_dim), self.dtype)
             ops.qk_norm_rope_append(qkv, s.n_heads, s.n_kv_heads, s.head_dim, self.q_gain, self.k_gain, eps,
                                     cos, sin, rot, q, cache.k, cache.v, cache.block_table, step.token_seq,
@@ -129,9 +140,7 @@ class Attention(Mixer):
                           s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, workspace=ws.scratch(),
                           cu_seqlens=step.cu_seqlens, max_new=step.max_new, q_counts=step.new_counts,
                           max_len=step.max_len, n_splits=self._decode_splits(step, cache))
-        splits = ops.gemm(o, self.w_o, x_accum, accumulate=True, workspace=ws.scratch(), defer=True)
-        if splits:
-            ws.set_pending(x_accum, splits)
+        ws.add_product(o, self.w_o, x_accum)
 
 
 register_mixer("attention", Attention)

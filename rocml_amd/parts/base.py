@@ -99,8 +99,22 @@ class Part:
         return 0
 
 
+@dataclass(frozen=True)
+class NormHint:
+    """A norm of the kind ``x / sqrt(mean(x^2) + eps) * gain`` over ``width`` values, as the
+    producer of ``x`` needs to know it to prepare the norm's output."""
+    gain: torch.Tensor
+    eps: float
+    width: int
+
+
 class Norm(Part):
     fuses_pending = False     # True: forward() takes ``pending`` partial sums and adds them to x itself
+
+    def prescale_hint(self) -> Optional[NormHint]:
+        """What the product that completes the residual stream needs to prepare this norm's output
+        up to the rows' scale; None if the norm is not of that kind."""
+        return None
 
     def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
         raise NotImplementedError
@@ -121,6 +135,12 @@ class PositionEncoding(Part):
 class Mixer(Part):
     adds_only = False     # True: forward() never reads x_accum, it only adds into it
 
+    def takes_row_scale(self, step: Any) -> bool:
+        """Whether, in this step, forward() can take its input as ``bfloat16(x * gain)`` with the
+        norm's row scale still to be applied (``step.row_scale``, an ``ops.RowScale``) instead of
+        the normed input."""
+        return False
+
     def cache_request(self) -> Optional[Any]:
         return None
 
@@ -134,6 +154,10 @@ class Mixer(Part):
 
 class FeedForward(Part):
     adds_only = False     # True: forward() never reads x_accum, it only adds into it
+
+    def takes_row_scale(self, step: Any) -> bool:
+        """As ``Mixer.takes_row_scale``."""
+        return False
 
     def forward(self, step: Any, xn: torch.Tensor, x_accum: torch.Tensor) -> None:
         raise NotImplementedError

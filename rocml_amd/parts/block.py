@@ -48,29 +48,56 @@ class PreNormBlock(Part):
         return n_tokens * self.hidden * size + self.mixer.activation_bytes(n_tokens) + self.ffn.activation_bytes(n_tokens)
 
     takes_pending = True      # forward() may be handed a stream that still lacks deferred sums
+    takes_next_norm = True    # forward() accepts the hint of the norm that reads the stream after it
 
-    def forward(self, step, x: torch.Tensor, cache, owns_cache: bool) -> None:
+    def entry_hint(self, step):
+        """The norm this block reads the residual stream with first, for the product that completes
+        the stream before it, if the block's mixer can apply the norm's scale itself in this step."""
+        return self._hint(step, self.mixer_norm, self.mixer)
+
+    def forward(self, step, x: torch.Tensor, cache, owns_cache: bool, next_norm=None) -> None:
+        """``next_norm``: the hint of the norm that reads ``x`` after this block (``entry_hint`` of
+        the block that runs next), or None."""
         ws = step.workspace
-        xn = ws.get("block.xn", tuple(x.shape), self.dtype)
-        self._norm(step, self.mixer_norm, x, xn)
+        xn, step.row_scale = self._norm(step, self.mixer_norm, x)
         if not getattr(self.mixer, "adds_only", False):
             ws.flush_pending()
+        ws.next_norm = self._hint(step, self.ffn_norm, self.ffn)
         self.mixer.forward(step, xn, x, cache, owns_cache)
-        self._norm(step, self.ffn_norm, x, xn)
+        ws.next_norm = None
+        xn, step.row_scale = self._norm(step, self.ffn_norm, x)
         if not getattr(self.ffn, "adds_only", False):
             ws.flush_pending()
+        ws.next_norm = next_norm
         self.ffn.forward(step, xn, x)
+        ws.next_norm = None
+        step.row_scale = None
 
     @staticmethod
-    def _norm(step, norm, x, xn) -> None:
-        """A part may leave the last step of its residual sum (adding split-K partial sums
-        to x) to the norm that reads x next; a norm that cannot do that gets x completed."""
+    def _hint(step, norm, consumer):
+        takes = getattr(consumer, "takes_row_scale", None)
+        hint = getattr(norm, "prescale_hint", None)
+        if takes is None or hint is None or not takes(step):
+            return None
+        return hint()
+
+    def _norm(self, step, norm, x):
+        """The norm's output and what is left to apply to it (None: nothing).  A part may leave the
+        last step of its residual sum (adding split-K partial sums to x) to the norm that reads x
+        next, or have prepared the norm's output itself; a norm that can use neither gets x
+        completed."""
         ws = step.workspace
+        gain = getattr(norm, "gain", None)
+        prepared = ws.take_prescaled(x, gain) if gain is not None else None
+        if prepared is not None:
+            return prepared
+        xn = ws.get("block.xn", tuple(x.shape), self.dtype)
         if getattr(norm, "fuses_pending", False):
             norm.forward(x, xn, pending=ws.take_pending(x))
         else:
             ws.flush_pending()
             norm.forward(x, xn)
+        return xn, None
 
 
 register_block("pre_norm", PreNormBlock)

@@ -46,20 +46,24 @@ class GatedMlp(FeedForward):
         fused = self.dtype == torch.bfloat16 and s.hidden % 8 == 0
         return n_tokens * s.intermediate * (size + (0 if fused else 8))
 
+    def takes_row_scale(self, step) -> bool:
+        # the gated epilogue of the few-rows products applies it
+        return self.w_gate_up is not None and self.fused and step.n_tokens <= ops.ROW_SCALE_MAX_ROWS
+
     def forward(self, step, xn, x_accum) -> None:
         s = self.spec
         n = step.n_tokens
         ws = step.workspace
         h = ws.get("mlp.h", (n, s.intermediate), self.dtype)
         if self.fused:
-            ops.gemm(xn, self.w_gate_up, h, workspace=ws.scratch(), epilogue="swiglu")
+            ops.gemm(xn, self.w_gate_up, h, workspace=ws.scratch(), epilogue="swiglu", row_scale=step.row_scale)
         else:
+            if step.row_scale is not None:
+                raise ConfigError("the feed-forward was handed an input without its norm's scale in a step it cannot scale")
             gate_up = ws.get("mlp.gate_up", (n, 2 * s.intermediate), torch.float32)
             ops.gemm(xn, self.w_gate_up, gate_up, workspace=ws.scratch())
             ops.swiglu(gate_up, h, interleaved=True)
-        splits = ops.gemm(h, self.w_down, x_accum, accumulate=True, workspace=ws.scratch(), defer=True)
-        if splits:
-            ws.set_pending(x_accum, splits)
+        ws.add_product(h, self.w_down, x_accum)
 
 
 register_feed_forward("gated_mlp", GatedMlp)

@@ -9,7 +9,7 @@ import torch
 
 from .. import ops
 from ..config.spec import NormSpec
-from .base import BuildContext, Norm, ParamSpec
+from .base import BuildContext, Norm, NormHint, ParamSpec
 from .registry import register_norm
 
 
@@ -26,6 +26,9 @@ class RMSNorm(Norm):
         self.gain = tensors["weight"]
 
     fuses_pending = True      # forward() can add a deferred product's partial sums to x itself
+
+    def prescale_hint(self) -> Optional[NormHint]:
+        return None if self.gain is None else NormHint(self.gain, self.eps, self.size)
 
     def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None,
                 pending: Optional[torch.Tensor] = None) -> None:

@@ -75,6 +75,8 @@ def _tensor_args_cost(skip: Tuple[int, ...] = (), flops_per_byte: float = 0.0) -
 # launch helper -> (label of the report row, bytes and flops of a call)
 _COSTS: Dict[str, Tuple[str, Callable]] = {
     "gemm": ("product", _gemm_cost),
+    "gemm_residual_prescale": ("product", lambda x, w, resid, gain, xg, ssq, *a, **kw: (
+        _nbytes(x, w, resid, resid, gain, xg, ssq), 2 * x.shape[0] * w.shape[0] * x.shape[1])),
     "attention": ("attention", _attention_cost),
     "attention_decode_fused": ("attention (norm, rotation, append)", _fused_attention_cost),
     "qk_norm_rope_append": ("q/k norm, rotation, append", _tensor_args_cost(skip=(11, 12))),   # not the whole cache

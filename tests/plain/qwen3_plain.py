@@ -23,13 +23,17 @@ def embedding(table: torch.Tensor, ids: Sequence[int]) -> torch.Tensor:
     return torch.stack([table[int(i)] for i in ids])
 
 
-def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, rounded_before_scale=None) -> torch.Tensor:
     """Per row: ``inv = 1/sqrt(sum(x^2)/n + eps)``, ``y_i = x_i * inv * w_i``; the
     gain multiplies directly, there is no ``1 + w``
-    (rocml-kernels/kernels/rmsnorm.hip:18-42)."""
+    (rocml-kernels/kernels/rmsnorm.hip:18-42).  ``rounded_before_scale`` (for the oracle of an
+    engine that stores ``x * w`` in low precision and applies the row's scale to the sums of
+    the product that follows) is applied to ``x * w``; the result is the same number otherwise."""
     n = x.shape[-1]
     mean_sq = (x * x).sum(dim=-1, keepdim=True) / n
     inv = 1.0 / torch.sqrt(mean_sq + eps)
+    if rounded_before_scale is not None:
+        return rounded_before_scale(x * weight) * inv
     return x * inv * weight
 
 
@@ -155,7 +159,7 @@ def layer_windows(cfg: dict) -> List[Optional[int]]:
 
 def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: Sequence[int],
             dtype: torch.dtype = torch.float64, first_position: int = 0, rounded=_same,
-            last: Optional[int] = None, rounded_probs=None) -> torch.Tensor:
+            last: Optional[int] = None, rounded_probs=None, ffn_norm_rounds_before_scale: bool = False) -> torch.Tensor:
     """Logits ``[T, V]`` at every position of one whole sequence.
 
     Pre-norm residual blocks (rocml/src/forward/chunk_forward.rs:96-135):
@@ -169,7 +173,9 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: Sequence[int],
     the attention's output and the gated activation; the residual stream, the norms'
     statistics, the rotation, the softmax statistics and all sums stay in ``dtype``.
     ``rounded_probs`` replaces it for the probabilities alone (``lambda t: t`` for an engine
-    whose attention multiplies probabilities and values in full precision)."""
+    whose attention multiplies probabilities and values in full precision).
+    ``ffn_norm_rounds_before_scale``: the norm before the feed-forward stores ``x * gain`` in
+    low precision and the row's scale reaches the gate and up sums unrounded."""
     w = {name: (rounded(t.to(dtype)) if t.dim() > 1 else t.to(dtype)) for name, t in weights.items()}
     eps = cfg["rms_norm_eps"]
     positions = [first_position + t for t in range(len(tokens))]
@@ -179,7 +185,10 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: Sequence[int],
         p = f"model.layers.{layer}."
         xn = rounded(rmsnorm(x, w[p + "input_layernorm.weight"], eps))
         x = x + attention_block(xn, w, p, cfg, positions, windows[layer], rounded, rounded_probs)
-        xn = rounded(rmsnorm(x, w[p + "post_attention_layernorm.weight"], eps))
+        if ffn_norm_rounds_before_scale:
+            xn = rmsnorm(x, w[p + "post_attention_layernorm.weight"], eps, rounded_before_scale=rounded)
+        else:
+            xn = rounded(rmsnorm(x, w[p + "post_attention_layernorm.weight"], eps))
         x = x + mlp_block(xn, w, p, rounded)
     if last is not None:            # logits of the last positions only (a large vocabulary)
         x = x[-last:]
