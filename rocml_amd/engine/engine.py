@@ -70,14 +70,21 @@ class Engine:
         self.cache.commit([slot], [new_len])
 
     # -- the step ------------------------------------------------------------------------
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], device_ids: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Runs the entries' tokens; returns ``[n_wanted, vocab]`` 32-bit logits on the
         device in the order of the entries and of their ``want`` lists, or None when
         nothing is wanted.  The result is a buffer of the engine and holds until the next
-        step."""
+        step.  ``device_ids`` (int32 on the device, one per entry, every entry bringing one
+        token): the token ids are taken from there instead of from the entries, whose tokens
+        only stand for their number; for ids that a sampler has just drawn and the host has not
+        seen yet."""
         spec = self.model.spec
         if not entries:
             return None
+        if device_ids is not None:
+            if any(len(e.tokens) != 1 for e in entries) or device_ids.numel() != len(entries) \
+                    or device_ids.dtype != torch.int32 or not device_ids.is_cuda:
+                raise RocmlError("ids on the device go with one token per entry: int32, one per entry")
         slots = [e.slot for e in entries]
         if len(set(slots)) != len(slots):
             raise RocmlError("a sequence appears twice in one step")
@@ -118,7 +125,7 @@ class Engine:
         if pieces is None:             # one piece: its reservation is all or nothing by itself
             self.cache.reserve(slots, new_lens)
             logits = self._run_piece(slots, starts, [list(e.tokens) for e in entries],
-                                     [list(e.want) for e in entries])
+                                     [list(e.want) for e in entries], device_ids)
             self.cache.commit(slots, new_lens)
             self.steps_run += 1
             return logits
@@ -166,7 +173,7 @@ class Engine:
         return pieces
 
     def _run_piece(self, slots: List[int], starts: List[int], tokens: List[List[int]],
-                   want: List[List[int]]) -> Optional[torch.Tensor]:
+                   want: List[List[int]], device_ids: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         ids, seq, pos, cu, lens, slot_arr = pack_step(slots, starts, tokens)
         want_rows = np.asarray([int(cu[b]) + w for b, ws_ in enumerate(want) for w in ws_], dtype=np.int32)
         width = _bucket(self.cache.table_width(slots))
@@ -176,6 +183,8 @@ class Engine:
         host = np.concatenate(parts) if parts else np.zeros(0, np.int32)
         meta = self.workspace.get("step.meta", (max(host.size, 1),), torch.int32)
         meta[:host.size].copy_(torch.from_numpy(host))
+        if device_ids is not None:
+            meta[:ids.size].copy_(device_ids)           # the ids lead the table
         max_new = max(len(t) for t in tokens)
         n_want = int(want_rows.size)
 

@@ -54,13 +54,23 @@ class GenerateStats:
 
 
 class EngineBackend:
-    """The loop's view of the engine and the sampler."""
+    """The loop's view of the engine and the sampler.
 
-    def __init__(self, engine, sampler=None):
+    With ``run_ahead`` (the default) the backend does not let the GPU wait for the host between
+    decode steps: as soon as the sampler has been launched it launches the next step for the same
+    sequences, with the token ids taken from the sampler's output on the device, and only then
+    waits for the ids to reach the host.  When the loop then asks for that step it is running
+    already; a sequence that the loop ended meanwhile (a stop token, a limit) was run one token
+    too far, which nobody sees: its row is dropped and its slot is released."""
+
+    def __init__(self, engine, sampler=None, run_ahead: bool = True):
         from ..sampling.sampler import DeviceSampler
         self.engine = engine
         self.sampler = sampler or DeviceSampler(engine.model.device)
         self.max_positions = engine.model.spec.max_positions
+        self.run_ahead = run_ahead and hasattr(self.sampler, "sample_start")
+        self._row_slots: Optional[List[int]] = None     # the slots whose logits the last step returned, row by row
+        self._ahead = None                              # (slots, logits, slots still live) of a step launched ahead
 
     def can_admit(self, lengths: Sequence[int], prompts: Optional[Sequence[int]] = None) -> bool:
         """Whether new sequences with prompts of ``prompts`` tokens that will grow to ``lengths``
@@ -79,17 +89,52 @@ class EngineBackend:
 
     def release(self, slot: int) -> None:
         self.engine.release(slot)
+        if self._ahead is not None:
+            self._ahead[2].discard(slot)        # the slot may come back as another sequence
 
     def step(self, slots: Sequence[int], tokens: Sequence[Sequence[int]]):
         from .batch import StepEntry
+        slots = list(slots)
+        ahead, self._ahead = self._ahead, None
+        if ahead is not None and all(len(t) == 1 for t in tokens) and set(slots) <= ahead[2]:
+            # the step is running already (with these tokens: they are what the sampler drew)
+            self._row_slots = slots
+            if slots == ahead[0]:
+                return ahead[1]
+            import torch
+            rows = torch.tensor([ahead[0].index(s) for s in slots], dtype=torch.int64, device=ahead[1].device)
+            return ahead[1].index_select(0, rows)
+        self._row_slots = slots
         return self.engine.step([StepEntry(s, list(t), [len(t) - 1]) for s, t in zip(slots, tokens)])
 
-    def sample(self, logits, seqs: Sequence[SequenceSampling]) -> List[int]:
-        return self.sampler.sample(logits, seqs)
+    def sample(self, logits, seqs: Sequence[SequenceSampling], may_continue: Optional[Sequence[bool]] = None) -> List[int]:
+        """``may_continue[b]``: whether sequence ``b`` goes on after this token unless it is a
+        stop token (the loop knows the limits); only those are run ahead."""
+        if not self.run_ahead or self._row_slots is None or len(self._row_slots) != len(seqs):
+            return self.sampler.sample(logits, seqs)
+        from .batch import StepEntry
+        started = self.sampler.sample_start(logits, seqs)
+        rows = [b for b in range(len(seqs)) if may_continue is None or may_continue[b]]
+        self._ahead = None
+        if rows:
+            slots = [self._row_slots[b] for b in rows]
+            ids = started[0]
+            if len(rows) != len(seqs):
+                import torch
+                ids = ids.index_select(0, torch.tensor(rows, dtype=torch.int64, device=ids.device))
+            try:
+                # those sequences one token further, as if none of them drew a stop token; refused (a
+                # full cache) it changes nothing and the loop goes on step by step
+                ahead = self.engine.step([StepEntry(s, [0], [0]) for s in slots], device_ids=ids)
+                self._ahead = (slots, ahead, set(slots))
+            except RocmlError:
+                self._ahead = None
+        return self.sampler.finish(started)
 
     def synchronize(self) -> None:
         import torch
-        torch.cuda.synchronize()
+        if torch.device(self.engine.model.device).type == "cuda":
+            torch.cuda.synchronize()
 
 
 @dataclass
@@ -109,6 +154,8 @@ class Generator:
         self.backend = backend
         self.max_batch = max_batch
         self.stats = GenerateStats()
+        import inspect
+        self._hints = "may_continue" in inspect.signature(backend.sample).parameters
         # called with the number of decode steps run so far after each of them: a place for a
         # benchmark to take its times without a loop of its own
         self.on_step = None
@@ -184,7 +231,13 @@ class Generator:
         self.stats.prompt_tokens += sum(len(s.request.prompt) for s in live)
         running = list(live)
         while running:
-            drawn = be.sample(logits, [s.sampling for s in running])
+            if self._hints:
+                # (a backend that runs ahead of the host wants to know who certainly ends here)
+                goes_on = [len(s.out) + 1 < s.request.max_new_tokens
+                           and len(s.request.prompt) + len(s.out) + 1 < be.max_positions for s in running]
+                drawn = be.sample(logits, [s.sampling for s in running], may_continue=goes_on)
+            else:
+                drawn = be.sample(logits, [s.sampling for s in running])
             still: List[_Live] = []
             for s, tok in zip(running, drawn):
                 reason = None

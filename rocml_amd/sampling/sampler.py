@@ -46,17 +46,33 @@ class DeviceSampler:
         self._ids_host: Optional[torch.Tensor] = None
 
     def _ids(self, out: torch.Tensor) -> List[int]:
+        return self.finish(self._start_copy(out))
+
+    def _start_copy(self, out: torch.Tensor):
         batch = out.numel()
         if self._ids_host is None or self._ids_host.numel() < batch:
             self._ids_host = torch.empty(max(batch, 64), dtype=torch.int32, pin_memory=True)
         host = self._ids_host[:batch]
         host.copy_(out, non_blocking=True)
-        torch.cuda.current_stream(self.device).synchronize()
+        done = torch.cuda.Event()
+        done.record(torch.cuda.current_stream(self.device))
+        return out, host, done
+
+    def finish(self, started) -> List[int]:
+        """Waits for the ids of ``sample_start`` to reach the host and returns them."""
+        _, host, done = started
+        done.synchronize()
         return host.tolist()
 
     def sample(self, logits: torch.Tensor, seqs: Sequence[SequenceSampling]) -> List[int]:
         """``logits`` is ``[B, V]`` 32-bit on the device, row ``b`` for ``seqs[b]``.  Returns
         the drawn ids and appends them to nothing: the caller decides what a token means."""
+        return self.finish(self.sample_start(logits, seqs))
+
+    def sample_start(self, logits: torch.Tensor, seqs: Sequence[SequenceSampling]):
+        """Launches the sampling and the copy of the drawn ids to the host without waiting for
+        either; ``finish`` waits.  The first element of what it returns is the ids on the device
+        (int32 ``[B]``), which work launched meanwhile may read."""
         batch, vocab = logits.shape
         assert batch == len(seqs)
         out = torch.empty(batch, dtype=torch.int32, device=self.device)
@@ -64,7 +80,7 @@ class DeviceSampler:
             if self._argmax_work is None or self._argmax_work.numel() < batch * ops.ARGMAX_WORK_WORDS:
                 self._argmax_work = torch.empty(max(batch, 64) * ops.ARGMAX_WORK_WORDS, dtype=torch.int32, device=self.device)
             ops.argmax(logits, out, self._argmax_work)
-            return self._ids(out)
+            return self._start_copy(out)
         if self._work is None or self._work.numel() < logits.numel():
             self._work = torch.empty(logits.numel(), dtype=torch.float32, device=self.device)
         window = max([s.params.repeat_penalty_window for s in seqs if s.params.penalty_active()] + [1])
@@ -101,4 +117,4 @@ class DeviceSampler:
                    top_k=dev[4 * batch:5 * batch], top_p=floats[2 * batch:3 * batch],
                    penalty=floats[3 * batch:4 * batch], history=dev[6 * batch:].view(batch, window),
                    history_len=dev[5 * batch:6 * batch], small_k=small_k)
-        return self._ids(out)
+        return self._start_copy(out)

@@ -177,3 +177,102 @@ def test_profiler_wraps_the_launch_helpers_only_while_it_is_active():
     assert profile.active() is None
     assert all(getattr(ops, name) is fn for name, fn in before.items())
     profile.set_phase("prefill")                     # without a profiler: nothing to tag
+
+
+# ---- the engine's backend running ahead of the host (no GPU: a scripted engine and sampler) -------
+class _FakeCache:
+    def __init__(self, slots):
+        self.free = list(range(slots))
+
+    class _Slots:
+        def __init__(self, outer):
+            self.outer = outer
+
+        @property
+        def n_free(self):
+            return len(self.outer.free)
+
+    @property
+    def slots(self):
+        return _FakeCache._Slots(self)
+
+    def fits(self, pieces, final=None):
+        return None
+
+
+class _FakeEngine:
+    """Next-token rule of ``Scripted``; a step may take its ids from a tensor 'on the device'."""
+
+    def __init__(self, slots=4, max_positions=1000):
+        import types
+        self.model = types.SimpleNamespace(spec=types.SimpleNamespace(max_positions=max_positions), device="cpu")
+        self.cache = _FakeCache(slots)
+        self.history = {}
+        self.steps = []
+
+    def plan_pieces(self, counts):
+        return [[(i, 0, c) for i, c in enumerate(counts)]]
+
+    def new_sequence(self):
+        s = self.cache.free.pop(0)
+        self.history[s] = []
+        return s
+
+    def release(self, slot):
+        del self.history[slot]
+        self.cache.free.insert(0, slot)
+
+    def step(self, entries, device_ids=None):
+        import torch
+        self.steps.append(([e.slot for e in entries], device_ids is not None))
+        rows = []
+        for i, e in enumerate(entries):
+            toks = [int(device_ids[i])] if device_ids is not None else list(e.tokens)
+            if len(self.history[e.slot]) + len(toks) > self.model.spec.max_positions:
+                raise RocmlError("context")
+            self.history[e.slot].extend(toks)
+            rows.append([float(sum(self.history[e.slot]) % 50)])
+        return torch.tensor(rows)
+
+
+class _FakeSampler:
+    def sample(self, logits, seqs):
+        return self.finish(self.sample_start(logits, seqs))
+
+    def sample_start(self, logits, seqs):
+        import torch
+        ids = logits[:, 0].to(torch.int32)
+        return ids, ids.clone(), None
+
+    def finish(self, started):
+        return started[1].tolist()
+
+
+@pytest.mark.parametrize("run_ahead", [True, False])
+def test_the_backend_may_run_ahead_of_the_host_without_changing_a_token(run_ahead):
+    from rocml_amd.engine.generate import EngineBackend
+    reqs = [Request([1, 2, 3], 5), Request([4], 2, stop_tokens=frozenset({9})), Request([7] * 6, 8), Request([9, 1], 1),
+            Request([5, 6], 10, stop_tokens=frozenset(_expected([5, 6], 10)[0][3:4])),
+            Request([3], 4), Request([8], 3), Request([2], 6)]               # prompts of one token on slots used before
+    want = Generator(Scripted(), max_batch=3).run(reqs)
+    engine = _FakeEngine(slots=3)
+    got = Generator(EngineBackend(engine, sampler=_FakeSampler(), run_ahead=run_ahead), max_batch=3).run(reqs)
+    assert [(r.tokens, r.finish_reason) for r in got] == [(r.tokens, r.finish_reason) for r in want]
+    assert not engine.history and sorted(engine.cache.free) == [0, 1, 2]
+    ahead = [slots for slots, from_device in engine.steps if from_device]
+    assert bool(ahead) == run_ahead
+    if run_ahead:
+        # a sequence is only run ahead when it may go on: the only tokens run for nothing are
+        # those behind a stop token (one request above stops on one)
+        ran = sum(len(s) for s in ahead)
+        useful = sum(len(r.tokens) - 1 for r in want if r.tokens)          # every token but the last is run through the model
+        assert useful <= ran <= useful + 2
+
+
+def test_running_ahead_stops_at_the_models_last_position():
+    from rocml_amd.engine.generate import EngineBackend
+    engine = _FakeEngine(slots=2, max_positions=6)
+    got = Generator(EngineBackend(engine, sampler=_FakeSampler()), max_batch=2).run([Request([1, 2, 3], 10), Request([4], 3)])
+    want = Generator(Scripted(max_positions=6), max_batch=2).run([Request([1, 2, 3], 10), Request([4], 3)])
+    assert [(r.tokens, r.finish_reason) for r in got] == [(r.tokens, r.finish_reason) for r in want]
+    assert got[0].finish_reason == "context" and all(len(h) <= 6 for h in engine.history.values())
