@@ -210,3 +210,60 @@ def test_a_windowed_group_takes_prompts_far_longer_than_its_window():
     c.free_sequence(b)
     assert c.fits([[("x", 256)], [("x", 512)]], final=[("x", 4096)]) is None
     assert c.fits([[("x", 256)]], final=[("x", 4097)]) is not None
+
+
+def test_a_cache_group_kind_of_its_own_needs_no_change_to_the_cache():
+    """A mixer with needs of its own (here: one narrow vector per position, in pages, beside a
+    counter per sequence) brings a request class and a group class and registers the pair; the
+    cache opens, commits, closes and checks it like its own kinds."""
+    from dataclasses import dataclass
+    from rocml_amd.cache import CacheLineView, PagedGroup, register_cache_group
+
+    @dataclass(frozen=True)
+    class LatentRequest:
+        width: int
+        window: int = None
+
+    class LatentGroup(PagedGroup):
+        def __init__(self, name, request, n_lines, geo):
+            super().__init__(name, request, n_lines, self.pool_pages(request.window, geo), geo.page_size, request.window)
+            self.latent = torch.zeros((n_lines, self.n_pages, geo.page_size, request.width), dtype=geo.dtype, device=geo.device)
+            self.tokens_seen = {}
+
+        @staticmethod
+        def planned_bytes(request, n_lines, geo):
+            return n_lines * PagedGroup.pool_pages(request.window, geo) * geo.page_size * request.width * 4
+
+        def open(self, slot):
+            super().open(slot)
+            self.tokens_seen[slot] = 0
+
+        def committed(self, slot, length):
+            super().committed(slot, length)
+            self.tokens_seen[slot] = length
+
+        def close(self, slot):
+            super().close(slot)
+            del self.tokens_seen[slot]
+
+        def view(self, line, step):
+            return CacheLineView(group=self, line=line, k=self.latent[line], block_table=step.block_tables[self.name])
+
+    register_cache_group(LatentRequest, LatentGroup)
+    from rocml_amd.cache.cache import planned_bytes
+    full = KVCacheRequest(n_kv_heads=1, head_dim=16)
+    reqs = [full, LatentRequest(24), LatentRequest(24), None, LatentRequest(24, window=100)]
+    assert planned_bytes(reqs, 64 * 10, torch.float32) == 2 * 640 * 16 * 4 + 2 * 640 * 24 * 4 + 640 * 24 * 4
+    c = Cache(reqs, max_tokens=64 * 10, dtype=torch.float32, device="cpu")
+    assert [g.name for g in c.kv_groups] == ["kv0", "latent0", "latent1w100"] and c.kv_groups[1].n_lines == 2
+    a, b = c.new_sequence(), c.new_sequence()
+    c.reserve([a, b], [200, 5])
+    c.commit([a, b], [200, 5])
+    latent = c.kv_groups[1]
+    assert latent.tokens_seen == {a: 200, b: 5} and len(latent.page_table(a)) == 4
+    assert c.kv_groups[2].page_table(a)[0] == -1                     # the windowed one gave its first page back
+    table = c.block_table(latent, [a, b], 4)
+    assert table.shape == (2, 4) and table[1, 1] == -1
+    c.free_sequence(a)
+    c.check()
+    assert latent.tokens_seen == {b: 5} and c.line(2)[0] is latent and c.line(2)[1] == 1
