@@ -261,8 +261,9 @@ ROCML_EXPORT int rocml_gemm_residual_prescale(const void* x, int ldx, const void
     if (m == 0) return 0;
     int tiles = ceil_div(n, 16);
     ROCML_REQUIRE(waves == 0 || waves == 4 || waves == 8 || waves == 16, "gemm_residual_prescale: 4, 8 or 16 waves, got %d", waves);
-    // waves: 0 = choose: eight a block when each still gets 512 of K, else four
-    if (waves == 0) waves = k >= 4096 ? 8 : 4;
+    // waves: 0 = choose: eight a block when each still gets 512 of K and the chip holds all blocks
+    // of eight at once, else four
+    if (waves == 0) waves = (k >= 4096 && tiles <= 256) ? 8 : 4;
 #define GRP_LAUNCH(W_)                                                                                          \
     gemm_residual_prescale_kernel<W_><<<tiles, 64 * W_, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw, resid, \
                                                                      ldr, gain, (bf16_t*)xg, ldg, ssq, tiles, m, n, k)
@@ -275,12 +276,19 @@ ROCML_EXPORT int rocml_gemm_residual_prescale(const void* x, int ldx, const void
 }
 
 // Whether rocml_gemm_residual_prescale is the faster way to add this product to the residual
-// stream and norm the result: its blocks own 16 columns and all of K, so the chip must hold them
-// in one round (256 CUs) and K must be short enough for the eight waves of a block (4096: measured
-// 11.6 us against 21.0 for the product cut along K over blocks plus the norm, at 4096 x 4096 and
-// 8 rows; with K of 12288 the two are equal, beyond that the cut product wins).
+// stream and norm the result.  Its blocks own 16 columns and all of K, so the chip (256 CUs) must
+// hold them in one round and K must be short enough for the waves of a block.  Measured against
+// the product cut along K over blocks plus the norm kernel: 4096 x 4096 at 8 rows 11.6 us against
+// 21.0; K of 12288 at 8 rows equal (25.7, 25.9), at 1 row 23.0 against 25.9; 5120 x 5120 (320
+// blocks of four waves, which the chip still holds at once) at 1 row 18.4 against 22.5, at 8 rows
+// equal; with longer K the cut product wins.
 ROCML_EXPORT int rocml_gemm_residual_prescale_pays(int m, int n, int k) {
-    return m >= 1 && m <= 16 && ceil_div(n, 16) <= 256 && k <= 4096 && k % 8 == 0;
+    if (m < 1 || m > 16 || k % 8 != 0) return 0;
+    int tiles = ceil_div(n, 16);
+    if (tiles <= 256 && k <= 4096) return 1;
+    if (m <= 2 && tiles <= 256 && k <= 12288) return 1;
+    if (m <= 2 && tiles <= 512 && k <= 5120) return 1;
+    return 0;
 }
 
 // algo: 0 = choose, 1 = plain tiled kernel, 2 = MFMA tile kernel, 3 = MFMA few-rows kernel (M <= 64),

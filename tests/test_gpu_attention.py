@@ -252,6 +252,38 @@ def test_decode_fused_with_norm_rotation_and_append(hq, hkv, d, lengths, qkv_spl
     _fused_case([(n, 1) for n in lengths], hq, hkv, d, qkv_splits, attn_splits, window, seed=11)
 
 
+def test_decode_fused_applies_a_row_scale():
+    """The projection's operand lacked its norm's scale: the kernel multiplies every sum of the
+    projection of token t by 1 / sqrt(sum of ssq[t] / width + eps) first.  Handing it the sums divided
+    by that number must give what the sums themselves give without a scale."""
+    hq, hkv, d, width = 8, 2, 128, 520
+    seqs = [(n, 1) for n in (1, 64, 65, 700, 129)]
+    n = len(seqs)
+    scale = 1.0 / math.sqrt(d)
+    g = torch.Generator().manual_seed(21)
+    for parts_per_row, qkv_splits in ((33, 1), (256, 3)):
+        ssq = torch.rand(n, parts_per_row, generator=g) * 5.0
+        eps = 1e-5
+        factor = 1.0 / torch.sqrt(ssq.double().sum(-1) / width + eps)            # per token
+        sums = torch.randn(qkv_splits, n, (hq + 2 * hkv) * d, generator=g) / math.sqrt(qkv_splits)
+        gains = [(1 + 0.3 * torch.randn(d, generator=g)).cuda() for _ in range(2)]
+        angle = torch.rand(n, d // 2, generator=g) * 6.28
+        cos, sin = torch.cos(angle).cuda(), torch.sin(angle).cuda()
+        ws = torch.empty(32 << 20, dtype=torch.uint8, device="cuda")
+        results = []
+        for lacking in (False, True):
+            dev, _, _, _ = _build(seqs, hq, hkv, d, torch.bfloat16, 22)
+            given = (sums.double() / factor[None, :, None]).float() if lacking else sums
+            given = given.cuda() if qkv_splits > 1 else given[0].cuda()
+            out = torch.full((n, hq * d), float("nan"), dtype=torch.bfloat16, device="cuda")
+            ops.attention_decode_fused(given, out, dev["kc"], dev["vc"], dev["table"], None, dev["tok_pos"], hq, hkv, d, scale,
+                                       gains[0], gains[1], eps, cos, sin, workspace=ws, max_len=700, n_splits=3,
+                                       row_scale=ops.RowScale(ssq.cuda(), eps, width) if lacking else None)
+            results.append((out.float().cpu(), dev["kc"].float().cpu(), dev["vc"].float().cpu()))
+        for a, b in zip(*results):
+            assert float((a - b).abs().max()) <= 1e-2 * float(a.abs().max())
+
+
 def test_decode_fused_without_norm_or_rotation():
     _fused_case([(77, 1), (200, 1)], 8, 4, 128, 2, 3, None, seed=12, norm=False)
     _fused_case([(77, 1), (200, 1)], 8, 4, 128, 1, 0, None, seed=13, rotate=False)

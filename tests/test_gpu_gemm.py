@@ -7,6 +7,7 @@ import torch
 pytestmark = pytest.mark.gpu
 
 from rocml_amd import ops  # noqa: E402
+from rocml_amd.errors import KernelError  # noqa: E402
 
 PLAIN, TILE, SKINNY, KPAR, TILE256, TILE192 = 1, 2, 3, 4, 5, 6
 
@@ -142,3 +143,60 @@ def test_many_rows_with_k_cut_in_pieces(m, n, k):
     out16 = torch.empty(m, n, dtype=torch.bfloat16, device="cuda")
     assert ops.gemm(x, w, out16, workspace=small, defer=True) == 0
     assert float((out16.double() - ref).abs().max()) < 5e-3 * scale
+
+
+@pytest.mark.parametrize("waves", [0, 4, 8])
+@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (3, 100, 72), (8, 4096, 1032), (16, 130, 4096), (7, 515, 264), (2, 88, 12288)])
+def test_residual_sum_that_prepares_the_next_norm(m, n, k, waves):
+    """resid += x W^T with whole sums, xg = bfloat16(resid * gain), and per 16 columns the sum of
+    squares of the new residual row, from which the consumer forms the norm's scale."""
+    x, w = _operands(m, n, k, torch.bfloat16, 5)
+    g = torch.Generator().manual_seed(6)
+    base = torch.randn(m, n, generator=g)
+    gain = 1 + 0.2 * torch.randn(n, generator=g)
+    resid = base.cuda()
+    xg = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    tiles = (n + ops.PRESCALE_TILE - 1) // ops.PRESCALE_TILE
+    ssq = torch.full((m, tiles), float("nan"), device="cuda")
+    assert ops.gemm_residual_prescale_fits(x, w)
+    ops.gemm_residual_prescale(x, w, resid, gain.cuda(), xg, ssq, waves=waves)
+    want = base.double() + _ref(x, w).cpu()
+    scale = max(1.0, float(want.abs().max()))
+    assert float((resid.double().cpu() - want).abs().max()) < 2e-5 * scale
+    assert float((xg.double().cpu() - want * gain.double()).abs().max()) < 5e-3 * float((want * gain.double()).abs().max())
+    padded = torch.zeros(m, tiles * 16, dtype=torch.float64)
+    padded[:, :n] = want ** 2
+    assert float((ssq.double().cpu() - padded.view(m, tiles, 16).sum(-1)).abs().max()) < 1e-5 * float(padded.max()) * 16
+    # the norm's output, put together the way a consumer does
+    eps = 1e-5
+    inv = 1.0 / torch.sqrt(ssq.double().cpu().sum(-1, keepdim=True) / n + eps)
+    normed = want / torch.sqrt((want ** 2).mean(-1, keepdim=True) + eps) * gain.double()
+    assert float((xg.double().cpu() * inv - normed).abs().max()) < 5e-3 * float(normed.abs().max())
+    with pytest.raises(KernelError):
+        ops.gemm_residual_prescale(torch.zeros(17, k, dtype=torch.bfloat16, device="cuda"), w,
+                                   torch.zeros(17, n, device="cuda"), gain.cuda(),
+                                   torch.zeros(17, n, dtype=torch.bfloat16, device="cuda"), torch.zeros(17, tiles, device="cuda"))
+
+
+@pytest.mark.parametrize("algo", [0, SKINNY, KPAR])
+@pytest.mark.parametrize("m,n,k,parts", [(1, 64, 64, 4), (2, 24576, 4096, 256), (8, 448, 96, 6), (16, 1000, 264, 17), (13, 300, 1032, 64)])
+def test_gated_epilogue_applies_a_row_scale(m, n, k, parts, algo):
+    """The operand lacks its norm's scale; the gated epilogue multiplies the sums of a row by
+    1 / sqrt(sum of the row's parts / K + eps) before the activation."""
+    x, w = _operands(m, n, k, torch.bfloat16, 7)
+    g = torch.Generator().manual_seed(8)
+    ssq = (torch.rand(m, parts, generator=g) * 3 * k / parts).cuda()
+    eps = 1e-5
+    inv = 1.0 / torch.sqrt(ssq.double().sum(-1, keepdim=True) / k + eps)
+    full = _ref(x, w) * inv
+    gate, up = full[:, 0::2], full[:, 1::2]
+    ref = gate / (1 + torch.exp(-gate)) * up
+    ws = torch.empty(16 << 20, dtype=torch.uint8, device="cuda")
+    out = torch.empty(m, n // 2, dtype=torch.bfloat16, device="cuda")
+    ops.gemm(x, w, out, algo=algo, workspace=ws, epilogue="swiglu", row_scale=ops.RowScale(ssq, eps, k))
+    assert float((out.double() - ref).abs().max()) < 5e-3 * max(1.0, float(ref.abs().max()))
+    with pytest.raises(KernelError):                       # not without the gated epilogue, not for more rows
+        ops.gemm(x, w, torch.empty(m, n, device="cuda"), workspace=ws, row_scale=ops.RowScale(ssq, eps, k))
+    with pytest.raises(KernelError):
+        ops.gemm(torch.zeros(17, k, dtype=torch.bfloat16, device="cuda"), w, torch.empty(17, n // 2, dtype=torch.bfloat16, device="cuda"),
+                 workspace=ws, epilogue="swiglu", row_scale=ops.RowScale(torch.ones(17, parts, device="cuda"), eps, k))
