@@ -97,8 +97,7 @@ def main() -> int:
         def step(self, slots, tokens):
             if all(len(t) == 1 for t in tokens):
                 return super().step(slots, tokens)
-            for s, t in zip(slots, tokens):
-                self.engine.adopt_positions(s, len(t))
+            self.engine.adopt_positions(slots, [len(t) for t in tokens])
             return torch.zeros((len(slots), spec.vocab), dtype=torch.float32, device=model.device)
 
     def decode(batch: int, steps: int, warmup: int):

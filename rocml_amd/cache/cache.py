@@ -395,15 +395,21 @@ class Cache:
     def length(self, slot: int) -> int:
         return self.lengths[slot]
 
-    def reserve(self, slots: Sequence[int], new_lens: Sequence[int]) -> None:
-        """Pages for every sequence to reach its new length, or none at all."""
-        for g in self.kv_groups:
+    def reserve(self, slots: Sequence[int], new_lens: Sequence[int], which: str = "all") -> None:
+        """Pages for every sequence to reach its new length, or none at all.  ``which``: ``all``
+        groups, only those that keep every position (``kept``) or only those with a window
+        (``windowed``): a step of several pieces takes the pages of the former for all its
+        sequences at once, so that they lie side by side in the pool as ``grow_together`` wants
+        them, and those of the latter piece by piece, between which such a group gives pages back."""
+        groups = [g for g in self.kv_groups
+                  if which == "all" or (g.window is None) == (which == "kept")]
+        for g in groups:
             need = sum(g.pages_needed(s, n) for s, n in zip(slots, new_lens))
             if need > g.n_free_pages:
                 raise CacheFullError(
                     f"cache group {g.name}: the step needs {need} more pages of {g.page_size} "
                     f"positions, {g.n_free_pages} of {g.n_pages} are free")
-        for g in self.kv_groups:
+        for g in groups:
             g.grow_together(slots, new_lens)
 
     def fits(self, pieces: Sequence[Sequence[Tuple[object, int]]],

@@ -724,6 +724,17 @@ gemm_residual_prescale_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_
         if (xrow) xd_[j] = *(const u32x4_t*)(in_ ? xp + (kb_) + j * 32 : xsafe); \
     }
     if (ks < ke) GR_LOAD(ks, wc, xc)
+    // The first wave finishes the block's outputs: what it needs of the residual stream and of the
+    // gain is asked for now, so that it has arrived when the sums are ready.
+    int n0 = tile * 16 + g * 4;
+    bool row_ok = col < m;
+    bool vec = row_ok && n0 + 3 < n && (ldr & 3) == 0 && (ldg & 3) == 0;
+    float4 r_old = make_float4(0.f, 0.f, 0.f, 0.f), gn = r_old;
+    if (wave == 0 && vec) {
+        r_old = *(const float4*)(resid + (size_t)col * ldr + n0);
+        gn = *(const float4*)(gain + n0);
+        asm volatile("" ::: "memory");          // (the loads stay here)
+    }
     for (int kb = ks; kb < ke; kb += GK_KC) {
         bool more = kb + GK_KC < ke;
         if (more) GR_LOAD(kb + GK_KC, wn, xn)
@@ -755,15 +766,11 @@ gemm_residual_prescale_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_
         for (int wv = 1; wv < WAVES; ++wv) sum += red[wv][lane][e];
         v[e] = sum;
     }
-    int n0 = tile * 16 + g * 4;
-    bool row_ok = col < m;
     float ss = 0.f;
-    if (row_ok && n0 + 3 < n && (ldr & 3) == 0 && (ldg & 3) == 0) {
-        float4* rp = (float4*)(resid + (size_t)col * ldr + n0);
-        float4 r = *rp;
-        float4 gn = *(const float4*)(gain + n0);
+    if (vec) {
+        float4 r = r_old;
         r.x += v[0]; r.y += v[1]; r.z += v[2]; r.w += v[3];
-        *rp = r;
+        *(float4*)(resid + (size_t)col * ldr + n0) = r;
         *(uint2*)(xg + (size_t)col * ldg + n0) = make_uint2(f32x2_to_bf16x2(r.x * gn.x, r.y * gn.y),
                                                              f32x2_to_bf16x2(r.z * gn.z, r.w * gn.w));
         ss = fmaf(r.x, r.x, fmaf(r.y, r.y, fmaf(r.z, r.z, r.w * r.w)));

@@ -58,16 +58,16 @@ class Engine:
     def length(self, slot: int) -> int:
         return self.cache.length(slot)
 
-    def adopt_positions(self, slot: int, n: int) -> None:
-        """Lengthens a sequence by ``n`` positions without running tokens: the cache rows are
+    def adopt_positions(self, slots: Sequence[int], counts: Sequence[int]) -> None:
+        """Lengthens sequences by ``counts`` positions without running tokens: the cache rows are
         whatever the pages held.  For measurements that want decode steps at a given depth
-        without paying for the prompt; results of such a sequence mean nothing."""
-        new_len = self.cache.length(slot) + n
-        if new_len > self.model.spec.max_positions:
-            raise ContextOverflowError(f"sequence would reach {new_len} positions; the model has "
+        without paying for the prompt; results of such sequences mean nothing."""
+        new_lens = [self.cache.length(s) + n for s, n in zip(slots, counts)]
+        if max(new_lens) > self.model.spec.max_positions:
+            raise ContextOverflowError(f"a sequence would reach {max(new_lens)} positions; the model has "
                                        f"{self.model.spec.max_positions}")
-        self.cache.reserve([slot], [new_len])
-        self.cache.commit([slot], [new_len])
+        self.cache.reserve(list(slots), new_lens)
+        self.cache.commit(list(slots), new_lens)
 
     # -- the step ------------------------------------------------------------------------
     def step(self, entries: Sequence[StepEntry], device_ids: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
@@ -134,6 +134,7 @@ class Engine:
         if n_want_total:
             result = torch.empty((n_want_total, spec.vocab), dtype=torch.float32, device=self.model.device)
         want_base = np.cumsum([0] + [len(e.want) for e in entries])
+        self.cache.reserve(slots, new_lens, which="kept")
         for piece in pieces:
             p_slots, p_starts, p_tokens, p_want, p_dest = [], [], [], [], []
             for i, lo, hi in piece:
@@ -145,7 +146,7 @@ class Engine:
                 p_want.append([w for _, w in wanted])
                 p_dest.extend(int(want_base[i]) + k for k, _ in wanted)
             p_lens = [s + len(t) for s, t in zip(p_starts, p_tokens)]
-            self.cache.reserve(p_slots, p_lens)
+            self.cache.reserve(p_slots, p_lens, which="windowed")
             logits = self._run_piece(p_slots, p_starts, p_tokens, p_want)
             if logits is not None:
                 result[torch.as_tensor(p_dest, device=self.model.device)] = logits

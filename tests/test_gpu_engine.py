@@ -80,6 +80,11 @@ def test_internal_cutting_of_long_steps_is_invisible(models, dtype):
     logits = engine.step([StepEntry(s, p, w) for s, p, w in zip(slots, prompts, want)]).cpu()
     expect = torch.cat([ref[w] for ref, w in zip(refs, want)])
     assert helpers.rel_to_max(logits, expect) < TOL[dtype]
+    # the group that keeps every position took its pages for the whole step at once, a page per
+    # sequence and round, however the step was cut: the sequences' first pages are neighbours
+    kept = [g for g in engine.cache.kv_groups if g.window is None][0]
+    first_pages = sorted(kept.page_table(s)[0] for s in slots)
+    assert first_pages[-1] - first_pages[0] == len(slots) - 1
     # the cache the pieces left is the one a whole step would leave: decode one more token each
     nxt = [7, 8, 9, 10]
     logits = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, nxt)]).cpu()
