@@ -6,7 +6,11 @@ resolves ``--model`` as a path if it looks like one, else as a catalog name,
 listing all names when it is unknown (rocml/src/registry/mod.rs:42-84,123-127).
 Here an entry carries the whole configuration, so a model with random weights
 needs no file.  Sizes of the 8B, 14B and 32B entries are the ones the
-benchmark configurations name; the two tiny entries are the test models.
+benchmark configurations name; the two tiny entries are the test models.  The
+reference's other dense names (0.6B, 1.7B, 4B; rocml/src/registry/catalog.rs:216-248)
+come without sizes in its files, which read them from each checkpoint: the sizes
+here are the ones published with those checkpoints and nothing in the reference
+pins them.
 """
 from __future__ import annotations
 
@@ -46,6 +50,12 @@ CATALOG: List[ModelEntry] = [
                default_ctx=128, init_norm_jitter=True),
     ModelEntry("tiny-b", _qwen3(384, 96, 224, 3, 6, 2, 32, 1000000.0, 1e-5, False, 512),
                default_ctx=512, init_norm_jitter=True),
+    ModelEntry("qwen3-0.6b", _qwen3(151936, 1024, 3072, 28, 16, 8, 128, 1000000.0, 1e-6, True, 40960),
+               sampling=QWEN_THINKING_SAMPLING),
+    ModelEntry("qwen3-1.7b", _qwen3(151936, 2048, 6144, 28, 16, 8, 128, 1000000.0, 1e-6, True, 40960),
+               sampling=QWEN_THINKING_SAMPLING),
+    ModelEntry("qwen3-4b", _qwen3(151936, 2560, 9728, 36, 32, 8, 128, 1000000.0, 1e-6, True, 40960),
+               sampling=QWEN_THINKING_SAMPLING),
     ModelEntry("qwen3-8b", _qwen3(151936, 4096, 12288, 36, 32, 8, 128, 1000000.0, 1e-6, False, 40960),
                sampling=QWEN_THINKING_SAMPLING),
     ModelEntry("qwen3-14b", _qwen3(151936, 5120, 17408, 40, 40, 8, 128, 1000000.0, 1e-6, False, 40960),

@@ -1,5 +1,6 @@
-"""Real layer sizes against the plain implementation: the Qwen3-8B and Qwen3-14B shapes of the
-catalog cut to their first two layers, with the real vocabulary, in 32-bit and in bfloat16;
+"""Real layer sizes against the plain implementation: the Qwen3-0.6B (tied output matrix, both
+norms of a decode layer prepared by the products before them), Qwen3-8B and Qwen3-14B shapes of
+the catalog cut to their first two layers, with the real vocabulary, in 32-bit and in bfloat16;
 an unequal batch whose last tokens are fed one by one.  The tiny configurations cannot show a
 fault that needs a width of 4096 or 5120, a head size of 128 with 32 or 40 heads, or a
 vocabulary of 151,936 (kernel choices, tile edges and split counts all depend on them)."""
@@ -16,7 +17,8 @@ TAIL = 4          # tokens fed one by one
 WANT = 8          # places compared per request: the last ones
 
 
-@pytest.mark.parametrize("name,lengths", [("qwen3-8b", [70, 333, 600]), ("qwen3-14b", [128, 257, 700])])
+@pytest.mark.parametrize("name,lengths", [("qwen3-0.6b", [40, 200, 333]), ("qwen3-8b", [70, 333, 600]),
+                                          ("qwen3-14b", [128, 257, 700])])
 def test_two_layers_of_a_real_shape(tmp_path, name, lengths):
     from rocml_amd.config.catalog import resolve
     from rocml_amd.engine import Engine, StepEntry
