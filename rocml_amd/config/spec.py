@@ -64,6 +64,26 @@ class GatedMlpSpec:
 
 
 @dataclass(frozen=True)
+class TokenTableSpec:
+    """The model's input: a row of a ``[vocab, hidden]`` table per token, times ``scale``."""
+    vocab: int
+    hidden: int
+    scale: float = 1.0
+    kind: str = "token_table"
+
+
+@dataclass(frozen=True)
+class NormLinearHeadSpec:
+    """The model's output: a norm of the wanted rows of the residual stream, then their
+    product with a ``[vocab, hidden]`` matrix; ``tied``: that matrix is the input's table."""
+    vocab: int
+    hidden: int
+    norm: NormSpec
+    tied: bool
+    kind: str = "norm_linear"
+
+
+@dataclass(frozen=True)
 class BlockSpec:
     """One layer: a mixer and a feed-forward with their norms.
 
@@ -98,6 +118,18 @@ class ModelSpec:
     max_positions: int
     embed_scale: float = 1.0
     eos_token_ids: Tuple[int, ...] = ()     # generation stops at any of these unless told otherwise
+    # The parts at the model's two ends, chosen by ``kind`` like every other part.  None: the token
+    # table and the norm-then-matrix head that the fields above describe.
+    embedding: Any = None
+    head: Any = None
+
+    def embedding_spec(self) -> Any:
+        return self.embedding if self.embedding is not None else \
+            TokenTableSpec(self.vocab, self.hidden, self.embed_scale)
+
+    def head_spec(self) -> Any:
+        return self.head if self.head is not None else \
+            NormLinearHeadSpec(self.vocab, self.hidden, self.final_norm, self.tie_lm_head)
 
     def validate(self) -> None:
         from ..errors import ConfigError

@@ -35,7 +35,7 @@ def _bucket(n: int) -> int:
 class Engine:
     def __init__(self, model: DecoderModel, max_tokens: int, max_seqs: Optional[int] = None,
                  max_step_tokens: int = 8192, use_graphs: bool = True):
-        if model.embed is None:
+        if not model.bound:
             raise RocmlError("the model has no weights bound")
         self.model = model
         if max_step_tokens < 1:

@@ -1,7 +1,7 @@
-"""A decoder built from a ``ModelSpec``: embedding, the layers in schedule order, final
-norm and output matrix.  It holds no sizes of its own and no knowledge of any
-architecture; the data flow is the reference's (rocml/src/forward/chunk_forward.rs:96-184):
-embedding, blocks, then norm and output product only for the rows whose logits are wanted.
+"""A decoder built from a ``ModelSpec``: an embedding part, the layers in schedule order and a
+head part.  It holds no sizes of its own and no knowledge of any architecture; the data flow
+is the reference's (rocml/src/forward/chunk_forward.rs:96-184): embedding, blocks, then the
+head (norm and output product) only for the rows whose logits are wanted.
 """
 from __future__ import annotations
 
@@ -9,12 +9,11 @@ from typing import Dict, List, Optional
 
 import torch
 
-from .. import ops
 from ..cache import Cache
 from ..cache.cache import HEADROOM_BYTES
 from ..config.spec import ModelSpec
 from ..errors import ConfigError
-from ..parts import BuildContext, ParamSpec, build_block, build_norm
+from ..parts import BuildContext, ParamSpec, build_block, build_embedding, build_head
 from .batch import StepContext
 from .workspace import Workspace
 
@@ -37,40 +36,44 @@ class DecoderModel:
         self.dtype = compute_dtype(dtype)
         self.device = torch.device(device)
         ctx = BuildContext(dtype=self.dtype, device=self.device)
+        self.embedding = build_embedding(spec.embedding_spec(), ctx)
         self.blocks = [build_block(b, ctx) for b in spec.layers]
-        self.final_norm = build_norm(spec.final_norm, ctx)
-        self.embed: Optional[torch.Tensor] = None
-        self.lm_head: Optional[torch.Tensor] = None
+        self.head = build_head(spec.head_spec(), ctx)
+        self.bound = False
         # whether a decode step may be recorded as a graph: every part must say so
-        self.graph_safe = all(getattr(b, "graph_safe", True) for b in self.blocks) and \
-            getattr(self.final_norm, "graph_safe", True)
+        self.graph_safe = all(getattr(part, "graph_safe", True)
+                              for part in [self.embedding, self.head] + self.blocks)
+
+    @property
+    def embed(self) -> Optional[torch.Tensor]:
+        """The embedding's table (None before weights are bound or if it has none)."""
+        return self.embedding.shared_matrix() if self.bound else None
+
+    @property
+    def lm_head(self) -> Optional[torch.Tensor]:
+        return getattr(self.head, "matrix", None)
 
     # -- parameters --------------------------------------------------------------------
     def param_specs(self) -> Dict[str, ParamSpec]:
-        s = self.spec
-        specs = {"embed.weight": ParamSpec((s.vocab, s.hidden))}
+        """Embedding parameters under ``embed.``, a layer's under ``layers.<i>.``, the head's under
+        the names it gives them."""
+        specs = {f"embed.{name}": p for name, p in self.embedding.param_specs().items()}
         for i, block in enumerate(self.blocks):
             for name, p in block.param_specs().items():
                 specs[f"layers.{i}.{name}"] = p
-        for name, p in self.final_norm.param_specs().items():
-            specs[f"final_norm.{name}"] = p
-        if not s.tie_lm_head:
-            specs["lm_head.weight"] = ParamSpec((s.vocab, s.hidden))
+        specs.update(self.head.param_specs())
         return specs
 
     def storage_dtype(self, p: ParamSpec) -> torch.dtype:
         return {"matrix": self.dtype, "gain": torch.float32, "int_table": torch.int32}[p.role]
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.embed = tensors["embed.weight"]
-        # A tied output matrix is the embedding table itself, one buffer
-        # (rocml/src/weights/mod.rs:48-62 loads it twice).
-        self.lm_head = self.embed if self.spec.tie_lm_head else tensors["lm_head.weight"]
+        self.embedding.bind({k[len("embed."):]: v for k, v in tensors.items() if k.startswith("embed.")})
         for i, block in enumerate(self.blocks):
             prefix = f"layers.{i}."
             block.bind({k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)})
-        self.final_norm.bind({k[len("final_norm."):]: v for k, v in tensors.items()
-                              if k.startswith("final_norm.")})
+        self.head.bind({k: tensors[k] for k in self.head.param_specs()}, shared=self.embedding.shared_matrix())
+        self.bound = True
 
     def weight_bytes(self) -> int:
         total = 0
@@ -92,8 +95,8 @@ class DecoderModel:
 
     def step_weight_bytes(self) -> int:
         """Bytes of weights a step has to read once: every layer as often as the schedule runs
-        it and the output matrix; of the embedding table only the step's rows, which are not
-        counted (a tied table is read as the output matrix)."""
+        it and the head's matrices; of the embedding only the step's rows, which are not
+        counted (a tied table is read as the head's matrix)."""
         per_layer = []
         for block in self.blocks:
             n = 0
@@ -104,13 +107,13 @@ class DecoderModel:
                 n += e * torch.empty((), dtype=self.storage_dtype(p)).element_size()
             per_layer.append(n)
         size = torch.empty((), dtype=self.dtype).element_size()
-        return sum(per_layer[e.layer] for e in self.spec.schedule) + self.spec.vocab * self.spec.hidden * size
+        return sum(per_layer[e.layer] for e in self.spec.schedule) + self.head.step_matrix_elements() * size
 
     def step_flops(self, new_counts, starts, n_wanted: int) -> int:
-        """Floating-point operations of a step: the layers in schedule order and the output
-        product for the wanted rows."""
+        """Floating-point operations of a step: the layers in schedule order and the head for
+        the wanted rows."""
         total = sum(self.blocks[e.layer].flops(new_counts, starts) for e in self.spec.schedule)
-        return total + 2 * n_wanted * self.spec.vocab * self.spec.hidden
+        return total + self.head.flops(n_wanted)
 
     # -- cache -------------------------------------------------------------------------
     def cache_requests(self) -> List[Optional[object]]:
@@ -122,10 +125,8 @@ class DecoderModel:
         """Bytes of activations and scratch memory a step of ``n_tokens`` tokens with ``n_wanted``
         rows of logits asks the workspace for: the residual stream, the largest layer's buffers
         (layers share theirs), the wanted rows and their logits, and the scratch memory."""
-        s = self.spec
-        size = torch.empty((), dtype=self.dtype).element_size()
         per_layer = max(b.activation_bytes(n_tokens) for b in self.blocks)
-        return (n_tokens * s.hidden * 4 + per_layer + n_wanted * (s.hidden * size + s.vocab * 4)
+        return (n_tokens * self.spec.hidden * 4 + per_layer + self.head.activation_bytes(n_wanted)
                 + Workspace.SCRATCH_BYTES)
 
     def new_cache(self, max_tokens: int, max_seqs: Optional[int] = None,
@@ -154,7 +155,7 @@ class DecoderModel:
         ws = step.workspace
         ws.drop_pending()
         x = ws.get("model.x", (step.n_tokens, s.hidden), torch.float32)
-        ops.embed_gather(self.embed, step.token_ids, x, s.embed_scale)
+        self.embedding.forward(step, x)
         for i, entry in enumerate(s.schedule):
             owner = i if entry.reads_cache_of is None else entry.reads_cache_of
             view = None
@@ -176,12 +177,6 @@ class DecoderModel:
         if n_want == 0:
             ws.drop_pending()
             return None
-        xn = ws.get("model.final_xn", (n_want, s.hidden), self.dtype)
-        if getattr(self.final_norm, "fuses_pending", False):
-            self.final_norm.forward(x, xn, rows=want_rows, pending=ws.take_pending(x))
-        else:
+        if not getattr(self.head, "takes_pending", False):
             ws.flush_pending()
-            self.final_norm.forward(x, xn, rows=want_rows)
-        logits = ws.get("model.logits", (n_want, s.vocab), torch.float32)
-        ops.gemm(xn, self.lm_head, logits, workspace=ws.scratch())
-        return logits
+        return self.head.forward(step, x, want_rows, n_want)

@@ -1,11 +1,11 @@
-from .base import (BuildContext, FeedForward, KVCacheRequest, Mixer, Norm, ParamSpec, Part,
+from .base import (BuildContext, Embedding, FeedForward, Head, KVCacheRequest, Mixer, Norm, ParamSpec, Part,
                    PositionEncoding, StateRequest)
-from .registry import (build_block, build_feed_forward, build_mixer, build_norm, build_position,
-                       register_block, register_feed_forward, register_mixer, register_norm,
-                       register_position)
-from . import rmsnorm, rope, attention, mlp, block  # noqa: F401  (register the built-in parts)
+from .registry import (build_block, build_embedding, build_feed_forward, build_head, build_mixer, build_norm,
+                       build_position, register_block, register_embedding, register_feed_forward,
+                       register_head, register_mixer, register_norm, register_position)
+from . import rmsnorm, rope, attention, mlp, block, embedding, head  # noqa: F401  (register the built-in parts)
 
-__all__ = ["BuildContext", "FeedForward", "KVCacheRequest", "Mixer", "Norm", "ParamSpec", "Part",
-           "PositionEncoding", "StateRequest", "build_block", "build_feed_forward", "build_mixer",
-           "build_norm", "build_position", "register_block", "register_feed_forward",
-           "register_mixer", "register_norm", "register_position"]
+__all__ = ["BuildContext", "Embedding", "FeedForward", "Head", "KVCacheRequest", "Mixer", "Norm", "ParamSpec",
+           "Part", "PositionEncoding", "StateRequest", "build_block", "build_embedding", "build_feed_forward",
+           "build_head", "build_mixer", "build_norm", "build_position", "register_block", "register_embedding",
+           "register_feed_forward", "register_head", "register_mixer", "register_norm", "register_position"]

@@ -10,7 +10,9 @@ layer is assembled from parts that know nothing about the model around them:
   storage in the cache (``cache_request``): keys and values, or a state of fixed size;
 * a **feed-forward** works on each token alone;
 * a **norm** maps the 32-bit residual stream to the activation type;
-* a **position encoding** prepares per-step tables that mixers share.
+* a **position encoding** prepares per-step tables that mixers share;
+* an **embedding** turns the step's token ids into the first residual stream, and a **head**
+  turns the wanted rows of the last one into logits.
 
 Mixers and feed-forwards add their result into the 32-bit residual stream they are
 handed (``x_accum``), which lets a product's epilogue do the residual sum.  A part whose
@@ -160,4 +162,38 @@ class FeedForward(Part):
         return False
 
     def forward(self, step: Any, xn: torch.Tensor, x_accum: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
+class Embedding(Part):
+    def shared_matrix(self) -> Optional[torch.Tensor]:
+        """The ``[vocab, hidden]`` table a head may use as its output matrix (tied weights), or
+        None if the embedding has no such table."""
+        return None
+
+    def forward(self, step: Any, x: torch.Tensor) -> None:
+        """Writes the residual stream's first value for the step's tokens into ``x`` (32-bit,
+        ``[tokens, hidden]``)."""
+        raise NotImplementedError
+
+
+class Head(Part):
+    takes_pending = False     # True: forward() may be handed a stream that still lacks deferred sums
+
+    def bind(self, tensors: Dict[str, torch.Tensor], shared: Optional[torch.Tensor] = None) -> None:
+        """``shared``: the embedding's table, for a head whose output matrix is tied to it."""
+
+    def step_matrix_elements(self) -> int:
+        """Elements of the matrices a step reads for its wanted rows (a tied table counts: the
+        head reads all of it, the embedding only the step's rows)."""
+        return self.matrix_elements()
+
+    def flops(self, n_wanted: int) -> int:
+        return 2 * n_wanted * self.step_matrix_elements()
+
+    def activation_bytes(self, n_wanted: int) -> int:
+        return 0
+
+    def forward(self, step: Any, x: torch.Tensor, want_rows: torch.Tensor, n_want: int) -> torch.Tensor:
+        """32-bit logits ``[n_want, vocab]`` of the token rows of ``x`` named by ``want_rows``."""
         raise NotImplementedError

@@ -11,7 +11,7 @@ from ..errors import ConfigError
 from .base import BuildContext
 
 _TABLES: Dict[str, Dict[str, Callable[[Any, BuildContext], Any]]] = {
-    "mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {},
+    "mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {}, "embedding": {}, "head": {},
 }
 
 
@@ -24,6 +24,8 @@ def register_feed_forward(kind, builder): _register("feed_forward", kind, builde
 def register_norm(kind, builder): _register("norm", kind, builder)
 def register_position(kind, builder): _register("position", kind, builder)
 def register_block(kind, builder): _register("block", kind, builder)
+def register_embedding(kind, builder): _register("embedding", kind, builder)
+def register_head(kind, builder): _register("head", kind, builder)
 
 
 def _build(table: str, kind: str, spec: Any, ctx: BuildContext) -> Any:
@@ -39,3 +41,5 @@ def build_feed_forward(spec, ctx): return _build("feed_forward", spec.kind, spec
 def build_norm(spec, ctx): return _build("norm", spec.kind, spec, ctx)
 def build_position(spec, ctx): return _build("position", spec.kind, spec, ctx)
 def build_block(spec, ctx): return _build("block", spec.arrangement, spec, ctx)
+def build_embedding(spec, ctx): return _build("embedding", spec.kind, spec, ctx)
+def build_head(spec, ctx): return _build("head", spec.kind, spec, ctx)

@@ -373,3 +373,108 @@ def test_toy_routed_feed_forward_and_toy_position_encoding():
     assert helpers.rel_to_max(helpers.run_tail_by_one(engine, b, 12), rb) < 1e-4
     got = helpers.run_batch(engine, [a, b], [35, 4])
     assert helpers.rel_to_max(got[0], ra) < 1e-4 and helpers.rel_to_max(got[1], rb) < 1e-4
+
+
+# ---- a toy embedding with learned positions and a toy head with a soft cap ------------------
+@dataclass(frozen=True)
+class PositionedTableSpec:
+    """Token row plus a learned row for the token's position: an additive position encoding."""
+    vocab: int
+    hidden: int
+    max_positions: int
+    kind: str = "toy_positioned_table"
+
+
+@dataclass(frozen=True)
+class CappedHeadSpec:
+    """Norm, product with a matrix of its own, then ``cap * tanh(logits / cap)``."""
+    vocab: int
+    hidden: int
+    eps: float
+    cap: float
+    kind: str = "toy_capped_head"
+
+
+def _toy_embedding_and_head():
+    from rocml_amd import ops
+    from rocml_amd.parts import Embedding, Head, ParamSpec, register_embedding, register_head
+
+    class PositionedTable(Embedding):
+        def __init__(self, spec, ctx):
+            self.spec = spec
+
+        def param_specs(self):
+            s = self.spec
+            return {"tokens.weight": ParamSpec((s.vocab, s.hidden)),
+                    "positions.weight": ParamSpec((s.max_positions, s.hidden))}
+
+        def bind(self, tensors):
+            self.tokens, self.positions = tensors["tokens.weight"], tensors["positions.weight"]
+
+        def forward(self, step, x):
+            ops.embed_gather(self.tokens, step.token_ids, x, 1.0)
+            x += self.positions.float()[step.token_pos.long()]
+
+    class CappedHead(Head):
+        def __init__(self, spec, ctx):
+            self.spec, self.dtype = spec, ctx.dtype
+
+        def param_specs(self):
+            s = self.spec
+            return {"out_norm.weight": ParamSpec((s.hidden,), role="gain", init="gain"),
+                    "out.weight": ParamSpec((s.vocab, s.hidden))}
+
+        def bind(self, tensors, shared=None):
+            self.gain, self.matrix = tensors["out_norm.weight"], tensors["out.weight"]
+
+        def forward(self, step, x, want_rows, n_want):
+            ws = step.workspace
+            xn = ws.get("toy_head.xn", (n_want, self.spec.hidden), self.dtype)
+            ops.rmsnorm(x, self.gain, self.spec.eps, xn, want_rows)
+            logits = ws.get("toy_head.logits", (n_want, self.spec.vocab), torch.float32)
+            ops.gemm(xn, self.matrix, logits, workspace=ws.scratch())
+            logits.copy_(self.spec.cap * torch.tanh(logits / self.spec.cap))
+            return logits
+
+    register_embedding("toy_positioned_table", PositionedTable)
+    register_head("toy_capped_head", CappedHead)
+
+
+def test_toy_embedding_with_learned_positions_and_toy_capped_head():
+    """The model's two ends are parts like the others: an embedding that adds a learned row per
+    position (attention then runs without rotation) and a head with a soft cap on the logits,
+    defined here and registered; the head does not declare that it takes deferred sums, so the
+    model completes the residual stream before it.  Decode steps are recorded and replayed."""
+    _toy_embedding_and_head()
+    hidden, vocab, d, cap = 40, 77, 16, 0.4
+    layers = [_block(hidden, _attention_spec(hidden, 4, 2, d, theta=None)) for _ in range(2)]
+    spec = ModelSpec(architecture="test", vocab=vocab, hidden=hidden, layers=tuple(layers),
+                     schedule=(ScheduleEntry(0), ScheduleEntry(1)), final_norm=NormSpec(hidden, 1e-5),
+                     tie_lm_head=False, max_positions=256,
+                     embedding=PositionedTableSpec(vocab, hidden, 256), head=CappedHeadSpec(vocab, hidden, 1e-5, cap))
+    for dtype, tol in (("float32", 1e-4), ("bfloat16", 3e-2)):
+        engine, w = _engine(spec, dtype, seed=11)
+        assert set(k for k in w if not k.startswith("layers.")) == \
+            {"embed.tokens.weight", "embed.positions.weight", "out_norm.weight", "out.weight"}
+
+        def reference(tokens):
+            t = len(tokens)
+            pos = list(range(t))
+            x = w["embed.tokens.weight"][tokens] + w["embed.positions.weight"][pos]
+            for i, b in enumerate(spec.layers):
+                pre = f"layers.{i}."
+                xn = plain.rmsnorm(x, w[pre + "mixer_norm.weight"], 1e-5)
+                x = x + plain_attention(xn, w, pre + "mixer.", b.mixer, pos)[0]
+                xn = plain.rmsnorm(x, w[pre + "ffn_norm.weight"], 1e-5)
+                x = x + plain.swiglu(xn @ w[pre + "ffn.gate_proj.weight"].t(), xn @ w[pre + "ffn.up_proj.weight"].t()) \
+                    @ w[pre + "ffn.down_proj.weight"].t()
+            logits = plain.rmsnorm(x, w["out_norm.weight"], 1e-5) @ w["out.weight"].t()
+            return cap * torch.tanh(logits / cap)
+
+        a, b = helpers.random_tokens(45, vocab, 12), helpers.random_tokens(21, vocab, 13)
+        ra, rb = reference(a), reference(b)
+        assert ra.abs().max() > 0.5 * cap                      # the cap bends the largest logits
+        assert helpers.rel_to_max(helpers.run_whole(engine, a), ra) < tol
+        assert helpers.rel_to_max(helpers.run_tail_by_one(engine, b, 12), rb) < tol
+        got = helpers.run_batch(engine, [a, b], [30, 5])
+        assert helpers.rel_to_max(got[0], ra) < tol and helpers.rel_to_max(got[1], rb) < tol
