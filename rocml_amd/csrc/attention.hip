@@ -52,7 +52,7 @@ static int launch_decode(const AttnArgs& a, hipStream_t stream) {
     // Enough blocks to fill the chip, at most one split per page of the longest sequence.
     int n_splits = a.n_splits_hint;
     if (n_splits <= 0) {
-        n_splits = 512 / (a.n_tokens * a.hkv);
+        n_splits = 2 * cu_count() / (a.n_tokens * a.hkv);
         int max_pages = (a.max_len + AM_PAGE - 1) / AM_PAGE;
         if (n_splits > max_pages) n_splits = max_pages;
     }

@@ -39,6 +39,20 @@ static int rocml_fail(const char* fmt, ...) {
 #define ROCML_LAST_ERROR_FN(family) \
     ROCML_EXPORT const char* family##_last_error() { return g_rocml_err; }
 
+// Compute units of the current device (256 on an MI355X).  Launch sizes are phrased in it: how
+// many blocks fill the chip, how many tiles leave CUs idle.
+static int cu_count() {
+    static int cached[64] = {0};
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 256;
+    if (cached[device] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || n <= 0) n = 256;
+        cached[device] = n;
+    }
+    return cached[device];
+}
+
 // ---- bf16 as raw 16 bits ------------------------------------------------------
 typedef uint16_t bf16_t;
 

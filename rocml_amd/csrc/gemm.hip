@@ -71,6 +71,7 @@ static int launch_mfma_tile(const void* x, int ldx, const void* w, int ldw, void
                             int n, int k, int shape, void* workspace, long long workspace_bytes, SplitPlan plan,
                             hipStream_t stream) {
     int splits = 1;
+    const int cus = cu_count();
     if (shape == 0) {
         double best = 1e30;
         // rows and columns of a tile, microseconds per 64-wide K stage, the shape's number
@@ -83,7 +84,7 @@ static int launch_mfma_tile(const void* x, int ldx, const void* w, int ldw, void
                                    (long long)pieces * m * n * (long long)sizeof(float) > workspace_bytes))
                     break;
                 long long blocks = tiles * pieces;
-                double per_cu = (double)ceil_div(blocks, 256);          // tiles of the busiest CU
+                double per_cu = (double)ceil_div(blocks, cus);          // tiles of the busiest CU
                 double stages = (double)ceil_div(ceil_div(k, pieces), GM_BK);
                 double t = per_cu * stages * kind.stage_us + 4.0;
                 if (pieces > 1) t += (double)pieces * m * n * 8.0 / 4.0e6;   // partial sums out and in, 4 TB/s
@@ -121,11 +122,14 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
         }
         ready = true;
     }
-    // (two waves per block also for the gated product of 17 to 32 rows: 9 % there)
+    // (two waves per block also for the gated product of 17 to 32 rows: 9 % there; "wide" is a
+    // product whose blocks of four waves alone are four to a CU or more)
     constexpr bool CAN_NARROW = MT <= 2;
-    bool narrow = MT == 1 ? (EPI == EPI_SWIGLU || n >= 65536) : (MT == 2 && EPI == EPI_SWIGLU);
+    const int cus = cu_count();
+    bool wide = n >= 256 * cus;
+    bool narrow = MT == 1 ? (EPI == EPI_SWIGLU || wide) : (MT == 2 && EPI == EPI_SWIGLU);
     int blocks_n = ceil_div(n, narrow ? 32 : 16 * WIDE);
-    int target = AHEAD ? 256 : 512;
+    int target = AHEAD ? cus : 2 * cus;
     int splits = target / blocks_n;
     int by_k = k / 512;
     if (splits > by_k) splits = by_k;
@@ -172,12 +176,12 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
 }
 
 // At most 16 rows: blocks of 16 weight rows, K split over the block's waves and, while there are
-// fewer than about 1000 blocks, over blocks as well (each wave keeps at least 256 of K).
+// fewer than four blocks a CU, over blocks as well (each wave keeps at least 256 of K).
 template <int EPI>
 static int launch_kpar(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m, int n, int k,
                        void* workspace, long long workspace_bytes, SplitPlan plan, hipStream_t stream) {
     int n_tiles = ceil_div(n, 16);
-    int splits = 1024 / n_tiles;
+    int splits = 4 * cu_count() / n_tiles;
     int by_k = k / 1024;
     if (splits > by_k) splits = by_k;
     if (splits > 16) splits = 16;
@@ -263,7 +267,7 @@ ROCML_EXPORT int rocml_gemm_residual_prescale(const void* x, int ldx, const void
     ROCML_REQUIRE(waves == 0 || waves == 4 || waves == 8 || waves == 16, "gemm_residual_prescale: 4, 8 or 16 waves, got %d", waves);
     // waves: 0 = choose: eight a block when each still gets 512 of K and the chip holds all blocks
     // of eight at once, else four
-    if (waves == 0) waves = (k >= 4096 && tiles <= 256) ? 8 : 4;
+    if (waves == 0) waves = (k >= 4096 && tiles <= cu_count()) ? 8 : 4;
 #define GRP_LAUNCH(W_)                                                                                          \
     gemm_residual_prescale_kernel<W_><<<tiles, 64 * W_, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw, resid, \
                                                                      ldr, gain, (bf16_t*)xg, ldg, ssq, tiles, m, n, k)
@@ -285,9 +289,10 @@ ROCML_EXPORT int rocml_gemm_residual_prescale(const void* x, int ldx, const void
 ROCML_EXPORT int rocml_gemm_residual_prescale_pays(int m, int n, int k) {
     if (m < 1 || m > 16 || k % 8 != 0) return 0;
     int tiles = ceil_div(n, 16);
-    if (tiles <= 256 && k <= 4096) return 1;
-    if (m <= 2 && tiles <= 256 && k <= 12288) return 1;
-    if (m <= 2 && tiles <= 512 && k <= 5120) return 1;
+    const int cus = cu_count();       // a block a CU, or two
+    if (tiles <= cus && k <= 4096) return 1;
+    if (m <= 2 && tiles <= cus && k <= 12288) return 1;
+    if (m <= 2 && tiles <= 2 * cus && k <= 5120) return 1;
     return 0;
 }
 
@@ -343,7 +348,8 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
         // Up to 16 rows the few-rows kernels; up to 64 rows still for the gated product (it cannot
         // cut K in pieces, which is what the tile kernel lives on with so few rows) and, up to 32
         // rows, for every product but the widest (the output projection over the vocabulary).
-        bool few_rows = m <= 16 || (m <= 64 && (gated || (m <= 32 && n < 65536)));
+        const int cus = cu_count();
+        bool few_rows = m <= 16 || (m <= 64 && (gated || (m <= 32 && n < 256 * cus)));
         bool skinny = algo == ALGO_MFMA_SKINNY || (algo == ALGO_AUTO && few_rows);
         SplitPlan plan{defer, deferred_splits, RowScale{row_ssq, row_parts, row_eps, 1.0f / (float)k}};
         int rc;
@@ -351,12 +357,13 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
         (epi == EPI_F32 ? fn<EPI_F32>(__VA_ARGS__)                   \
          : epi == EPI_BF16 ? fn<EPI_BF16>(__VA_ARGS__)               \
          : epi == EPI_ACC ? fn<EPI_ACC>(__VA_ARGS__) : fn<EPI_SWIGLU>(__VA_ARGS__))
-        // One or two rows: the kernel whose waves split K, unless the output is narrow (4096 or
-        // 5120 wide, the products that return to the hidden size): its blocks of 16 weight rows
-        // are then so few that K must be cut across blocks as well and a wave is left with one
-        // chunk; the few-rows kernel is 10 to 15 % faster there.  Beyond two rows the activations
+        // One or two rows: the kernel whose waves split K, unless the output is narrow (fewer than
+        // one and a half blocks of 16 weight rows a CU: 4096 or 5120 wide on 256 CUs, the products
+        // that return to the hidden size): its blocks are then so few that K must be cut across
+        // blocks as well and a wave is left with one chunk; the few-rows kernel is 10 to 15 %
+        // faster there.  Beyond two rows the activations
         // read from L2 cost more than the block sharing of the few-rows kernel.
-        bool kpar = algo == ALGO_MFMA_KPAR || (algo == ALGO_AUTO && m <= 2 && n >= 6144);
+        bool kpar = algo == ALGO_MFMA_KPAR || (algo == ALGO_AUTO && m <= 2 && 2 * (n / 16) >= 3 * cus);
         if (kpar) rc = BY_EPI(launch_kpar, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
         else if (skinny) rc = BY_EPI(launch_skinny_m, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
         else rc = BY_EPI(launch_mfma_tile, x, ldx, w, ldw, out, ldo, m, n, k,

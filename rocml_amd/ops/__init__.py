@@ -92,6 +92,20 @@ def _check(family: str, status: int) -> None:
         raise KernelError(msg)
 
 
+_cus = {}
+
+
+def cu_count(device) -> int:
+    """Compute units of ``device`` (256 on an MI355X, which is also the answer for a device that is
+    not a GPU, where parts are built only to be counted); launch sizes are phrased in it."""
+    device = torch.device(device)
+    if device.type != "cuda":
+        return 256
+    if device not in _cus:
+        _cus[device] = int(torch.cuda.get_device_properties(device).multi_processor_count)
+    return _cus[device]
+
+
 def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 

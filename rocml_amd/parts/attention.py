@@ -36,6 +36,7 @@ class Attention(Mixer):
             raise ConfigError(f"window must be positive, got {spec.window}")
         self.spec = spec
         self.dtype = ctx.dtype
+        self.n_cus = ops.cu_count(ctx.device)
         self.q_dim = spec.n_heads * spec.head_dim
         self.kv_dim = spec.n_kv_heads * spec.head_dim
         self.position = build_position(spec.position, ctx) if spec.position is not None else None
@@ -100,7 +101,7 @@ class Attention(Mixer):
         if step.max_new != 1:
             return 0
         blocks = step.n_tokens * self.spec.n_kv_heads
-        return max(1, min(512 // blocks, cache.block_table.shape[1], 64))
+        return max(1, min(2 * self.n_cus // blocks, cache.block_table.shape[1], 64))
 
     def forward(self, step, xn, x_accum, cache, owns_cache: bool) -> None:
         s = self.spec
