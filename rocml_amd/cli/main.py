@@ -10,7 +10,6 @@ import argparse
 import json
 import statistics
 import sys
-import time
 from typing import List, Optional
 
 from ..errors import RocmlError
