@@ -99,6 +99,46 @@ static int launch_mfma_tile(const void* x, int ldx, const void* w, int ldw, void
     return launch_mfma_tile_as<EPI, GemmTile128>(x, ldx, w, ldw, out, ldo, m, n, k, splits, workspace, plan, stream);
 }
 
+// The kernel for 17 to 64 rows on a product that cannot be cut along K (the gated product), with
+// WAVES waves a block, each on 16 columns.
+template <int MT, int EPI, int WAVES>
+static int launch_ahead_whole(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m, int n,
+                              int k, hipStream_t stream) {
+    constexpr int LDS = 2 * MT * 16 * GS_ROW * 16;
+    static bool ready = false;
+    if (!ready) {
+        if (allow_lds(gemm_skinny_ahead_kernel<MT, EPI, false, WAVES>, LDS, "gemm")) return 1;
+        ready = true;
+    }
+    gemm_skinny_ahead_kernel<MT, EPI, false, WAVES><<<dim3(ceil_div(n, 16 * WAVES), 1), 64 * WAVES, LDS, stream>>>(
+        (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, round_up(k, GS_KC));
+    return 0;
+}
+
+// Waves a block for such a product.  A CU pulls weight rows in 64-byte runs at a limited rate (the
+// kernel's loads put a row's four pieces into the lanes of one instruction) and a second block on
+// a CU stages the activations again, so the blocks should be one round that uses every CU: the
+// fewest waves whose blocks the chip holds at once.  Measured at 64 rows: 24576 columns in 44 us
+// with six waves (256 blocks; eight waves are 192 blocks and leave a quarter of 256 CUs idle:
+// 49 us; five are two rounds: 72), 34816 x 5120 in 79 us with nine (eight: 116), 51200 x 5120 in
+// 115 us with sixteen (eight: 124).  ``skip_from..skip_to``: counts whose kernel does not fit its
+// registers.  A product wider than one round of the largest blocks gets the count that leaves the
+// fewest columns on the busiest CU.
+static int ahead_waves(int n, int cus, int skip_from, int skip_to) {
+    for (int waves = 2; waves <= 16; ++waves)
+        if ((waves < skip_from || waves > skip_to) && ceil_div(n, 16 * waves) <= cus) return waves;
+    int best = 16, best_cols = 1 << 30;
+    for (int waves = 16; waves >= 2; --waves) {
+        if (waves >= skip_from && waves <= skip_to) continue;
+        int cols = ceil_div(ceil_div(n, 16 * waves), cus) * 16 * waves;
+        if (cols < best_cols) {
+            best = waves;
+            best_cols = cols;
+        }
+    }
+    return best;
+}
+
 template <int MT, int EPI>
 static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m, int n,
                          int k, void* workspace, long long workspace_bytes, SplitPlan plan, hipStream_t stream) {
@@ -108,7 +148,8 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
     // number), about 512 blocks.  Beyond 16 rows the kernel that requests two steps ahead, with
     // eight waves per block (LDS for the activations limits a CU to two blocks at 64 rows;
     // eight waves double the weight bytes in flight per CU and halve the times the activations
-    // are read), about 256 blocks.
+    // are read), about 256 blocks; the gated product, which cannot be cut along K, gets the
+    // number of waves that makes its blocks one round (ahead_waves).
     constexpr bool AHEAD = MT > 1;
     constexpr int WIDE = AHEAD ? 8 : 4;
     static bool ready = false;
@@ -122,12 +163,10 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
         }
         ready = true;
     }
-    // (two waves per block also for the gated product of 17 to 32 rows: 9 % there; "wide" is a
-    // product whose blocks of four waves alone are four to a CU or more)
-    constexpr bool CAN_NARROW = MT <= 2;
+    // ("wide" is a product whose blocks of four waves alone are four to a CU or more)
     const int cus = cu_count();
     bool wide = n >= 256 * cus;
-    bool narrow = MT == 1 ? (EPI == EPI_SWIGLU || wide) : (MT == 2 && EPI == EPI_SWIGLU);
+    bool narrow = MT == 1 && (EPI == EPI_SWIGLU || wide);
     int blocks_n = ceil_div(n, narrow ? 32 : 16 * WIDE);
     int target = AHEAD ? cus : 2 * cus;
     int splits = target / blocks_n;
@@ -143,17 +182,25 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
     splits = ceil_div(k, k_per_split);
     dim3 grid(blocks_n, splits);
     if (splits == 1 && narrow) {
-        if constexpr (CAN_NARROW && AHEAD)
-            gemm_skinny_ahead_kernel<MT, EPI, false, 2><<<grid, 128, LDS, stream>>>(
-                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
-        else if constexpr (CAN_NARROW)
+        if constexpr (MT == 1)
             gemm_skinny_kernel<MT, EPI, false, 2><<<grid, 128, LDS, stream>>>(
                 (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split, plan.rs);
     } else if (splits == 1) {
-        if constexpr (AHEAD)
+        if constexpr (AHEAD && EPI == EPI_SWIGLU) {
+            // (at 49 to 64 rows the kernels of 13 to 15 waves need more registers than 832 to 960
+            // threads leave each)
+            switch (ahead_waves(n, cus, MT == 4 ? 13 : 17, MT == 4 ? 15 : 17)) {
+#define AHEAD_CASE(W_) case W_: return launch_ahead_whole<MT, EPI, W_>(x, ldx, w, ldw, out, ldo, m, n, k, stream);
+                AHEAD_CASE(2) AHEAD_CASE(3) AHEAD_CASE(4) AHEAD_CASE(5) AHEAD_CASE(6) AHEAD_CASE(7) AHEAD_CASE(8)
+                AHEAD_CASE(9) AHEAD_CASE(10) AHEAD_CASE(11) AHEAD_CASE(12) AHEAD_CASE(13) AHEAD_CASE(14)
+                AHEAD_CASE(15) AHEAD_CASE(16)
+#undef AHEAD_CASE
+                default: return rocml_fail("gemm: no kernel of that many waves");
+            }
+        } else if constexpr (AHEAD) {
             gemm_skinny_ahead_kernel<MT, EPI, false, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
                 (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
-        else
+        } else
             gemm_skinny_kernel<MT, EPI, false, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
                 (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split, plan.rs);
     } else {

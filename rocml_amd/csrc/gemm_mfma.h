@@ -480,9 +480,10 @@ gemm_skinny_ahead_kernel(const bf16_t* x, int ldx, const bf16_t* w, int ldw, voi
     extern __shared__ u32x4_t gs_smem[];              // [2][MT*16][GS_ROW]
     constexpr int ROWS = MT * 16;
     constexpr int THREADS = 64 * WAVES;
-    constexpr int XL = ROWS * (GS_KC / 8) / THREADS;  // activation loads per thread and step
+    constexpr int XPIECES = ROWS * (GS_KC / 8);       // 16-byte pieces of the activations per step
+    constexpr int XL = (XPIECES + THREADS - 1) / THREADS;   // loads per thread and step
+    constexpr bool XEXACT = XPIECES % THREADS == 0;   // else the last round has threads without a piece
     constexpr int D = 2;                              // steps that the weights are requested ahead
-    static_assert(XL >= 1 && ROWS * (GS_KC / 8) % THREADS == 0, "activation pieces must divide among the threads");
     int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     int block_row = blockIdx.x * (16 * WAVES);
     int n0 = block_row + wave * 16;
@@ -501,6 +502,7 @@ gemm_skinny_ahead_kernel(const bf16_t* x, int ldx, const bf16_t* w, int ldw, voi
         int piece = tid + i * THREADS;
         xk[i] = (piece % (GS_KC / 8)) * 8;
         xoff[i] = ((uint32_t)(piece / (GS_KC / 8)) * (uint32_t)ldx + xk[i]) * 2;
+        if (!XEXACT && piece >= XPIECES) xk[i] = 0x40000000;     // beyond every K range: never loaded
     }
     u32x4_t wr[D][8], xr[2][XL];
     f32x4_t acc[MT];
@@ -542,7 +544,8 @@ gemm_skinny_ahead_kernel(const bf16_t* x, int ldx, const bf16_t* w, int ldw, voi
         u32x4_t* sx_ = gs_smem + (set_) * ROWS * GS_ROW;                                        \
         _Pragma("unroll") for (int i = 0; i < XL; ++i) {                                        \
             int piece_ = tid + i * THREADS;                                                     \
-            sx_[(piece_ / (GS_KC / 8)) * GS_ROW + piece_ % (GS_KC / 8)] = xr[set_][i];          \
+            if (XEXACT || piece_ < XPIECES)                                                     \
+                sx_[(piece_ / (GS_KC / 8)) * GS_ROW + piece_ % (GS_KC / 8)] = xr[set_][i];      \
         }                                                                                       \
     }
     GA_LOAD_X(0, 0)
