@@ -103,7 +103,7 @@ static int launch_mfma_tile(const void* x, int ldx, const void* w, int ldw, void
 // WAVES waves a block, each on 16 columns.
 template <int MT, int EPI, int WAVES>
 static int launch_ahead_whole(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m, int n,
-                              int k, hipStream_t stream) {
+                              int k, RowScale rs, hipStream_t stream) {
     constexpr int LDS = 2 * MT * 16 * GS_ROW * 16;
     static bool ready = false;
     if (!ready) {
@@ -111,7 +111,7 @@ static int launch_ahead_whole(const void* x, int ldx, const void* w, int ldw, vo
         ready = true;
     }
     gemm_skinny_ahead_kernel<MT, EPI, false, WAVES><<<dim3(ceil_div(n, 16 * WAVES), 1), 64 * WAVES, LDS, stream>>>(
-        (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, round_up(k, GS_KC));
+        (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, round_up(k, GS_KC), rs);
     return 0;
 }
 
@@ -142,14 +142,28 @@ static int ahead_waves(int n, int cus, int skip_from, int skip_to) {
 template <int MT, int EPI>
 static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m, int n,
                          int k, void* workspace, long long workspace_bytes, SplitPlan plan, hipStream_t stream) {
+    const int cus = cu_count();
+    if constexpr (EPI == EPI_SWIGLU) {
+        // The gated epilogue needs whole sums: the kernel that requests two steps ahead, whatever
+        // the number of rows, with the number of waves that makes its blocks one round.  (At 49 to
+        // 64 rows the kernels of 13 to 15 waves need more registers than 832 to 960 threads
+        // leave each.)
+        switch (ahead_waves(n, cus, MT == 4 ? 13 : 17, MT == 4 ? 15 : 17)) {
+#define AHEAD_CASE(W_) case W_: return launch_ahead_whole<MT, EPI, W_>(x, ldx, w, ldw, out, ldo, m, n, k, plan.rs, stream);
+            AHEAD_CASE(2) AHEAD_CASE(3) AHEAD_CASE(4) AHEAD_CASE(5) AHEAD_CASE(6) AHEAD_CASE(7) AHEAD_CASE(8)
+            AHEAD_CASE(9) AHEAD_CASE(10) AHEAD_CASE(11) AHEAD_CASE(12) AHEAD_CASE(13) AHEAD_CASE(14)
+            AHEAD_CASE(15) AHEAD_CASE(16)
+#undef AHEAD_CASE
+            default: return rocml_fail("gemm: no kernel of that many waves");
+        }
+    } else {
     constexpr int LDS = 2 * MT * 16 * GS_ROW * 16;
     // Up to 16 rows: four waves per block, or two for the wide products that cannot be split
     // (more, smaller blocks keep more loads in flight when nothing else multiplies their
     // number), about 512 blocks.  Beyond 16 rows the kernel that requests two steps ahead, with
     // eight waves per block (LDS for the activations limits a CU to two blocks at 64 rows;
     // eight waves double the weight bytes in flight per CU and halve the times the activations
-    // are read), about 256 blocks; the gated product, which cannot be cut along K, gets the
-    // number of waves that makes its blocks one round (ahead_waves).
+    // are read), about 256 blocks.
     constexpr bool AHEAD = MT > 1;
     constexpr int WIDE = AHEAD ? 8 : 4;
     static bool ready = false;
@@ -164,16 +178,14 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
         ready = true;
     }
     // ("wide" is a product whose blocks of four waves alone are four to a CU or more)
-    const int cus = cu_count();
-    bool wide = n >= 256 * cus;
-    bool narrow = MT == 1 && (EPI == EPI_SWIGLU || wide);
+    bool narrow = MT == 1 && n >= 256 * cus;
     int blocks_n = ceil_div(n, narrow ? 32 : 16 * WIDE);
     int target = AHEAD ? cus : 2 * cus;
     int splits = target / blocks_n;
     int by_k = k / 512;
     if (splits > by_k) splits = by_k;
     if (splits > 16) splits = 16;
-    if (splits < 1 || EPI == EPI_SWIGLU || narrow) splits = 1;     // the gated epilogue needs whole sums
+    if (splits < 1 || narrow) splits = 1;
     long long per_split = (long long)m * n * sizeof(float);
     if (splits > 1 && (long long)splits * per_split > workspace_bytes)
         splits = workspace ? (int)(workspace_bytes / per_split) : 1;
@@ -184,32 +196,21 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
     if (splits == 1 && narrow) {
         if constexpr (MT == 1)
             gemm_skinny_kernel<MT, EPI, false, 2><<<grid, 128, LDS, stream>>>(
-                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split, plan.rs);
+                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
     } else if (splits == 1) {
-        if constexpr (AHEAD && EPI == EPI_SWIGLU) {
-            // (at 49 to 64 rows the kernels of 13 to 15 waves need more registers than 832 to 960
-            // threads leave each)
-            switch (ahead_waves(n, cus, MT == 4 ? 13 : 17, MT == 4 ? 15 : 17)) {
-#define AHEAD_CASE(W_) case W_: return launch_ahead_whole<MT, EPI, W_>(x, ldx, w, ldw, out, ldo, m, n, k, stream);
-                AHEAD_CASE(2) AHEAD_CASE(3) AHEAD_CASE(4) AHEAD_CASE(5) AHEAD_CASE(6) AHEAD_CASE(7) AHEAD_CASE(8)
-                AHEAD_CASE(9) AHEAD_CASE(10) AHEAD_CASE(11) AHEAD_CASE(12) AHEAD_CASE(13) AHEAD_CASE(14)
-                AHEAD_CASE(15) AHEAD_CASE(16)
-#undef AHEAD_CASE
-                default: return rocml_fail("gemm: no kernel of that many waves");
-            }
-        } else if constexpr (AHEAD) {
+        if constexpr (AHEAD)
             gemm_skinny_ahead_kernel<MT, EPI, false, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
                 (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
-        } else
+        else
             gemm_skinny_kernel<MT, EPI, false, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
-                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split, plan.rs);
+                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, out, ldo, m, n, k, k_per_split);
     } else {
         if constexpr (AHEAD)
             gemm_skinny_ahead_kernel<MT, EPI, true, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
                 (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, workspace, n, m, n, k, k_per_split);
         else
             gemm_skinny_kernel<MT, EPI, true, WIDE><<<grid, 64 * WIDE, LDS, stream>>>(
-                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, workspace, n, m, n, k, k_per_split, RowScale{});
+                (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, workspace, n, m, n, k, k_per_split);
         if (plan.defer && ldo == n) {
             // the caller's next kernel adds the partial sums itself
             *plan.deferred = splits;
@@ -220,6 +221,7 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
             (const float*)workspace, out, ldo, m, n, splits);
     }
     return 0;
+    }
 }
 
 // At most 16 rows: blocks of 16 weight rows, K split over the block's waves and, while there are
@@ -404,13 +406,14 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
         (epi == EPI_F32 ? fn<EPI_F32>(__VA_ARGS__)                   \
          : epi == EPI_BF16 ? fn<EPI_BF16>(__VA_ARGS__)               \
          : epi == EPI_ACC ? fn<EPI_ACC>(__VA_ARGS__) : fn<EPI_SWIGLU>(__VA_ARGS__))
-        // One or two rows: the kernel whose waves split K, unless the output is narrow (fewer than
+        // One or two rows (but not the gated product, which has its own choice of blocks): the
+        // kernel whose waves split K, unless the output is narrow (fewer than
         // one and a half blocks of 16 weight rows a CU: 4096 or 5120 wide on 256 CUs, the products
         // that return to the hidden size): its blocks are then so few that K must be cut across
         // blocks as well and a wave is left with one chunk; the few-rows kernel is 10 to 15 %
         // faster there.  Beyond two rows the activations
         // read from L2 cost more than the block sharing of the few-rows kernel.
-        bool kpar = algo == ALGO_MFMA_KPAR || (algo == ALGO_AUTO && m <= 2 && 2 * (n / 16) >= 3 * cus);
+        bool kpar = algo == ALGO_MFMA_KPAR || (algo == ALGO_AUTO && m <= 2 && !gated && 2 * (n / 16) >= 3 * cus);
         if (kpar) rc = BY_EPI(launch_kpar, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
         else if (skinny) rc = BY_EPI(launch_skinny_m, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
         else rc = BY_EPI(launch_mfma_tile, x, ldx, w, ldw, out, ldo, m, n, k,

@@ -107,6 +107,60 @@ __device__ __forceinline__ float row_scale_finish(RowScale rs, int lane, int m, 
     return (lane & 15) < m ? 1.0f / sqrtf(s * rs.inv_width + rs.eps) : 1.0f;
 }
 
+// The same scales formed by several waves, each for NR rows of its own from row0 (4 or 8: fewer
+// loads in flight per lane, for kernels whose registers are taken by weights on their way):
+// scale_out[row0 .. row0 + NR) in LDS; red: NR x RS_RED_STRIDE floats that the wave has to itself.
+template <int NR>
+__device__ __forceinline__ void row_scale_rows(RowScale rs, int lane, int m, int row0, float* red, float* scale_out) {
+    static_assert(NR == 4 || NR == 8, "four or eight rows a wave");
+    if (!rs.ssq) {
+        if (lane < NR) scale_out[row0 + lane] = 1.0f;
+        return;
+    }
+    float part[NR];
+#pragma unroll
+    for (int i = 0; i < NR; ++i) part[i] = 0.f;
+    // (no branch between the loads of different rows, as in row_scale_request)
+    if ((rs.parts & 3) == 0) {
+        int chunks = rs.parts / 4;
+        const float4* all = (const float4*)rs.ssq;
+        for (int base = 0; base < chunks; base += 64) {
+            bool ok = base + lane < chunks;
+            int c = ok ? base + lane : 0;
+            float4 v[NR];
+#pragma unroll
+            for (int i = 0; i < NR; ++i) v[i] = all[(size_t)min(row0 + i, m - 1) * chunks + c];
+#pragma unroll
+            for (int i = 0; i < NR; ++i) part[i] += ok ? (v[i].x + v[i].y) + (v[i].z + v[i].w) : 0.f;
+        }
+    } else {
+        for (int base = 0; base < rs.parts; base += 64) {
+            bool ok = base + lane < rs.parts;
+            int p = ok ? base + lane : 0;
+            float v[NR];
+#pragma unroll
+            for (int i = 0; i < NR; ++i) v[i] = rs.ssq[(size_t)min(row0 + i, m - 1) * rs.parts + p];
+#pragma unroll
+            for (int i = 0; i < NR; ++i) part[i] += ok ? v[i] : 0.f;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NR; ++i) red[i * RS_RED_STRIDE + lane] = part[i];
+    __builtin_amdgcn_wave_barrier();
+    constexpr int LPR = 64 / NR;                      // lanes that share a row, NR values each
+    int i = lane / LPR, sub = lane % LPR;
+    const float4* mine = (const float4*)(red + i * RS_RED_STRIDE + sub * NR);
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < NR / 4; ++j) {
+        float4 v = mine[j];
+        s += (v.x + v.y) + (v.z + v.w);
+    }
+#pragma unroll
+    for (int off = 1; off < LPR; off <<= 1) s += __shfl_xor(s, off, 64);
+    if (sub == 0) scale_out[row0 + i] = row0 + i < m ? 1.0f / sqrtf(s * rs.inv_width + rs.eps) : 1.0f;
+}
+
 template <int EPI>
 __device__ __forceinline__ void epilogue_store(void* out, size_t idx, float v) {
     if (EPI == EPI_F32) ((float*)out)[idx] = v;
@@ -353,7 +407,7 @@ __device__ __forceinline__ void skinny_epilogue(const f32x4_t (&acc)[MT], void* 
 template <int MT, int EPI, bool PARTIAL, int WAVES = 4>
 __global__ void __launch_bounds__(64 * WAVES)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw,
-                   void* __restrict__ out, int ldo, int m, int n, int k, int k_per_split, RowScale rs) {
+                   void* __restrict__ out, int ldo, int m, int n, int k, int k_per_split) {
     extern __shared__ u32x4_t gs_smem[];              // [2][MT*16][GS_ROW]
     constexpr int ROWS = MT * 16;
     constexpr int THREADS = 64 * WAVES;
@@ -406,19 +460,6 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restri
 
     GS_LOAD_W(0, wcur)
     GS_LOAD_X(0)
-    // The rows' scales, if the operand lacks them (only the gated epilogue of at most 16 rows
-    // applies them): the block's first wave forms them while the first weights are on their way
-    // and leaves them in LDS for the epilogue.  (Held in registers through the loop they cost the
-    // kernel a wave per SIMD; asked for in the epilogue, a trip to memory at the kernel's end.)
-    constexpr bool SCALES = MT == 1 && EPI == EPI_SWIGLU && !PARTIAL;
-    __shared__ float gs_scale[16];
-    __shared__ __attribute__((aligned(16))) float gs_red[SCALES ? 16 * RS_RED_STRIDE : 4];
-    if (SCALES && wave == 0) {
-        float scale_part[16];
-        row_scale_request(rs, lane, m, scale_part);
-        float mine = row_scale_finish(rs, lane, m, scale_part, gs_red);
-        if (lane < 16) gs_scale[lane] = mine;
-    }
     GS_STORE_X(0, 0)
     __syncthreads();
     for (int c = 0; c < n_chunks; ++c) {
@@ -449,8 +490,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restri
 #undef GS_LOAD_W
 #undef GS_LOAD_X
 #undef GS_STORE_X
-    float row_scale = SCALES ? gs_scale[lane & 15] : 1.0f;
-    skinny_epilogue<MT, EPI, PARTIAL>(acc, out, ldo, m, n, n0, lane, blockIdx.y, row_scale);
+    skinny_epilogue<MT, EPI, PARTIAL>(acc, out, ldo, m, n, n0, lane, blockIdx.y);
 }
 
 // The same product for 17 to 64 rows.  With more rows a step costs more (four products and four
@@ -476,7 +516,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t ga_buffer(const void* base, lo
 template <int MT, int EPI, bool PARTIAL, int WAVES>
 __global__ void __launch_bounds__(64 * WAVES)
 gemm_skinny_ahead_kernel(const bf16_t* x, int ldx, const bf16_t* w, int ldw, void* out, int ldo, int m, int n,
-                         int k, int k_per_split) {
+                         int k, int k_per_split, RowScale rs = RowScale{}) {
     extern __shared__ u32x4_t gs_smem[];              // [2][MT*16][GS_ROW]
     constexpr int ROWS = MT * 16;
     constexpr int THREADS = 64 * WAVES;
@@ -556,6 +596,15 @@ gemm_skinny_ahead_kernel(const bf16_t* x, int ldx, const bf16_t* w, int ldw, voi
     GA_KEEP_ORDER
     GA_LOAD_W(1, 1)
     GA_KEEP_ORDER
+    // The rows' scales, if the operand lacks them (the gated epilogue of at most 16 rows applies
+    // them): the block's first waves form them, four rows each, while the first weights are on
+    // their way and leave them in LDS for the epilogue.
+    constexpr bool SCALES = MT == 1 && EPI == EPI_SWIGLU && !PARTIAL;
+    __shared__ float ga_scale[16];
+    __shared__ __attribute__((aligned(16))) float ga_red[SCALES ? 16 * RS_RED_STRIDE : 4];
+    constexpr int SCALE_WAVES = WAVES >= 4 ? 4 : 2, SCALE_ROWS = 16 / SCALE_WAVES;
+    if (SCALES && wave < SCALE_WAVES)
+        row_scale_rows<SCALE_ROWS>(rs, lane, m, wave * SCALE_ROWS, ga_red + wave * SCALE_ROWS * RS_RED_STRIDE, ga_scale);
     GA_STORE_X(0)
     __syncthreads();
     for (int c0 = 0; c0 < n_steps; c0 += D) {
@@ -592,7 +641,8 @@ gemm_skinny_ahead_kernel(const bf16_t* x, int ldx, const bf16_t* w, int ldw, voi
 #undef GA_LOAD_W
 #undef GA_LOAD_X
 #undef GA_STORE_X
-    skinny_epilogue<MT, EPI, PARTIAL>(acc, out, ldo, m, n, n0, lane, blockIdx.y);
+    float row_scale = SCALES ? ga_scale[lane & 15] : 1.0f;
+    skinny_epilogue<MT, EPI, PARTIAL>(acc, out, ldo, m, n, n0, lane, blockIdx.y, row_scale);
 }
 
 // ---- at most 16 rows -------------------------------------------------------------------------
