@@ -139,6 +139,74 @@ static int ahead_waves(int n, int cus, int skip_from, int skip_to) {
     return best;
 }
 
+// The same kernel on one K range of a product that is cut along K: 32-bit partial sums
+// [split][M][N] into the workspace.
+template <int MT, int WAVES>
+static int launch_ahead_split(const void* x, int ldx, const void* w, int ldw, void* workspace, int m, int n, int k,
+                              int splits, int k_per_split, hipStream_t stream) {
+    constexpr int LDS = 2 * MT * 16 * GS_ROW * 16;
+    static bool ready = false;
+    if (!ready) {
+        if (allow_lds(gemm_skinny_ahead_kernel<MT, EPI_F32, true, WAVES>, LDS, "gemm")) return 1;
+        ready = true;
+    }
+    gemm_skinny_ahead_kernel<MT, EPI_F32, true, WAVES><<<dim3(ceil_div(n, 16 * WAVES), splits), 64 * WAVES, LDS, stream>>>(
+        (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, workspace, n, m, n, k, k_per_split);
+    return 0;
+}
+
+// Blocks of a product that may be cut along K: waves a block (16 columns each) and K pieces, so
+// that the CU with the most work has as little as possible: its weight bytes (rounds of blocks
+// times a block's columns times its K range) plus its share of the partial sums, which are
+// written once and read once.  6144 x 4096 at 8 rows: 64 blocks of six waves times four pieces are
+// one round of 256 equal blocks; 96 blocks of four waves times four pieces leave half the CUs with
+// two blocks and half with one.
+struct BlockChoice { int waves, splits, k_per_split; };
+
+// An estimate of the busiest CU's time in microseconds.  A wave keeps two steps of weights
+// (16 KB) on their way for the two microseconds a trip takes, a CU pulls such rows at up to about
+// 45 GB/s however many waves ask (measured: 2.9 us more per 16 columns x 4096 a CU), a block
+// stages its rows' activations of its K range through LDS once, LDS holds so many blocks of these
+// rows at a time, and the partial sums are written here and read by the next kernel.
+static double block_cost(BlockChoice c, int m, int row_tiles, int n, int cus) {
+    const double lds_block = 2.0 * row_tiles * 16 * GS_ROW * 16;
+    const int resident = (int)(160.0 * 1024 / lds_block) < 1 ? 1 : (int)(160.0 * 1024 / lds_block);
+    long long blocks = (long long)ceil_div(n, 16 * c.waves) * c.splits;
+    int per_cu = (int)ceil_div(blocks, (long long)cus);
+    int together = per_cu < resident ? per_cu : resident;
+    double rounds = (double)ceil_div(per_cu, together);
+    double rate = 8.0e3 * c.waves * together;                              // bytes per microsecond
+    if (rate > 45.0e3) rate = 45.0e3;
+    double weights = 16.0 * c.waves * c.k_per_split * 2.0 * together;      // of the blocks that run together
+    double staged = 16.0 * row_tiles * c.k_per_split * 2.0 * together;
+    double cost = rounds * (weights / rate + staged / 100.0e3 + 3.0);
+    if (c.splits > 1) cost += (double)c.splits * (m * (double)n * 8.0 / 2.0e6 + 0.15);
+    return cost;
+}
+
+static BlockChoice choose_blocks(BlockChoice usual, int m, int row_tiles, int n, int k, int cus,
+                                 long long workspace_bytes, int skip_from, int skip_to) {
+    BlockChoice best = usual;
+    double best_cost = 1e30;
+    for (int kps = GS_KC; kps < k + GS_KC; kps += GS_KC) {
+        int splits = ceil_div(k, kps);
+        if (splits > 16) continue;
+        if (splits > 1 && (kps < 2 * GS_KC || (long long)splits * m * n * (long long)sizeof(float) > workspace_bytes)) continue;
+        for (int waves = 2; waves <= 16; ++waves) {
+            if (waves >= skip_from && waves <= skip_to) continue;
+            BlockChoice c{waves, splits, kps};
+            double cost = block_cost(c, m, row_tiles, n, cus);
+            if (cost < best_cost * 0.999) {
+                best_cost = cost;
+                best = c;
+            }
+        }
+    }
+    // the usual blocks (four or eight waves, about two blocks or one a CU) unless the estimate
+    // promises a clear gain: it is rough, and they are what the kernels were tuned with
+    return best_cost < 0.93 * block_cost(usual, m, row_tiles, n, cus) ? best : usual;
+}
+
 template <int MT, int EPI>
 static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m, int n,
                          int k, void* workspace, long long workspace_bytes, SplitPlan plan, hipStream_t stream) {
@@ -193,6 +261,30 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
     int k_per_split = round_up(ceil_div(k, splits), GS_KC);
     splits = ceil_div(k, k_per_split);
     dim3 grid(blocks_n, splits);
+    if (!narrow && workspace) {
+        BlockChoice usual{WIDE, splits, k_per_split};
+        BlockChoice c = choose_blocks(usual, m, MT, n, k, cus, workspace_bytes, MT == 4 ? 13 : 17, MT == 4 ? 15 : 17);
+        if (c.splits > 1 && (c.waves != usual.waves || c.splits != usual.splits)) {
+            int rc = 1;
+            switch (c.waves) {
+#define AHEAD_CASE(W_) case W_: rc = launch_ahead_split<MT, W_>(x, ldx, w, ldw, workspace, m, n, k, c.splits, c.k_per_split, stream); break;
+                AHEAD_CASE(2) AHEAD_CASE(3) AHEAD_CASE(4) AHEAD_CASE(5) AHEAD_CASE(6) AHEAD_CASE(7) AHEAD_CASE(8)
+                AHEAD_CASE(9) AHEAD_CASE(10) AHEAD_CASE(11) AHEAD_CASE(12) AHEAD_CASE(13) AHEAD_CASE(14)
+                AHEAD_CASE(15) AHEAD_CASE(16)
+#undef AHEAD_CASE
+                default: return rocml_fail("gemm: no kernel of that many waves");
+            }
+            if (rc) return rc;
+            if (plan.defer && ldo == n) {
+                *plan.deferred = c.splits;
+                return 0;
+            }
+            long long total = (long long)m * n;
+            gemm_splitk_reduce_kernel<EPI><<<ceil_div(total, 256), 256, 0, stream>>>(
+                (const float*)workspace, out, ldo, m, n, c.splits);
+            return 0;
+        }
+    }
     if (splits == 1 && narrow) {
         if constexpr (MT == 1)
             gemm_skinny_kernel<MT, EPI, false, 2><<<grid, 128, LDS, stream>>>(
