@@ -200,3 +200,51 @@ def test_gated_epilogue_applies_a_row_scale(m, n, k, parts, algo):
     with pytest.raises(KernelError):
         ops.gemm(torch.zeros(17, k, dtype=torch.bfloat16, device="cuda"), w, torch.empty(17, n // 2, dtype=torch.bfloat16, device="cuda"),
                  workspace=ws, epilogue="swiglu", row_scale=ops.RowScale(torch.ones(17, parts, device="cuda"), eps, k))
+
+
+@pytest.mark.parametrize("m", [3, 16, 20, 40, 64])
+@pytest.mark.parametrize("n,k", [(34816, 264), (51200, 512), (65568, 256), (90, 2056)])
+def test_wide_gated_products_take_blocks_of_many_waves(m, n, k):
+    """The gated product runs on blocks of as many waves as make one round over the chip: nine at
+    34816 columns, thirteen (sixteen at 49 to 64 rows) at 51200, and beyond one round of sixteen
+    waves the count that leaves the busiest CU the fewest columns; with and without a row scale."""
+    x, w = _operands(m, n, k, torch.bfloat16, 11)
+    full = _ref(x, w)
+    ws = torch.empty(16 << 20, dtype=torch.uint8, device="cuda")
+    out = torch.empty(m, n // 2, dtype=torch.bfloat16, device="cuda")
+    for scaled in (False, True):
+        if scaled and m > ops.ROW_SCALE_MAX_ROWS:
+            continue
+        inv = 1.0
+        scale = None
+        if scaled:
+            ssq = (torch.rand(m, 5, generator=torch.Generator().manual_seed(12)) * k).cuda()
+            inv = 1.0 / torch.sqrt(ssq.double().sum(-1, keepdim=True) / k + 1e-6)
+            scale = ops.RowScale(ssq, 1e-6, k)
+        gate, up = (full * inv)[:, 0::2], (full * inv)[:, 1::2]
+        ref = gate / (1 + torch.exp(-gate)) * up
+        out.fill_(float("nan"))
+        ops.gemm(x, w, out, workspace=ws, epilogue="swiglu", row_scale=scale)
+        assert float((out.double() - ref).abs().max()) < 5e-3 * max(1.0, float(ref.abs().max()))
+
+
+@pytest.mark.parametrize("m", [5, 16, 24, 32])
+@pytest.mark.parametrize("n,k", [(6144, 4096), (7168, 5120), (5120, 5120), (1000, 3080), (4096, 4096)])
+def test_few_rows_products_with_chosen_blocks(m, n, k):
+    """A product cut along K whose waves a block and K pieces are chosen for the busiest CU (six
+    waves and four pieces at 6144 x 4096, seven at 7168 x 5120, five at 5120 x 5120), complete or
+    with its partial sums left to the caller."""
+    x, w = _operands(m, n, k, torch.bfloat16, 13)
+    ref = _ref(x, w)
+    tol = 2e-5 * max(1.0, float(ref.abs().max()))
+    ws = torch.empty(32 << 20, dtype=torch.uint8, device="cuda")
+    base = torch.randn(m, n, device="cuda")
+    out = base.clone()
+    ops.gemm(x, w, out, accumulate=True, workspace=ws)
+    assert float((out.double() - (ref + base.double())).abs().max()) < tol
+    splits = ops.gemm(x, w, out, workspace=ws, defer=True)
+    if splits:
+        partials = ws[:splits * m * n * 4].view(torch.float32).view(splits, m, n)
+        assert float((partials.double().sum(0) - ref).abs().max()) < tol
+    else:
+        assert float((out.double() - ref).abs().max()) < tol
