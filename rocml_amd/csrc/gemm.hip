@@ -421,20 +421,21 @@ ROCML_EXPORT int rocml_gemm_residual_prescale(const void* x, int ldx, const void
 }
 
 // Whether rocml_gemm_residual_prescale is the faster way to add this product to the residual
-// stream and norm the result.  Its blocks own 16 columns and all of K, so the chip (256 CUs) must
-// hold them in one round and K must be short enough for the waves of a block.  Measured against
-// the product cut along K over blocks plus the norm kernel: 4096 x 4096 at 8 rows 11.6 us against
-// 21.0; K of 12288 at 8 rows equal (25.7, 25.9), at 1 row 23.0 against 25.9; 5120 x 5120 (320
-// blocks of four waves, which the chip still holds at once) at 1 row 18.4 against 22.5, at 8 rows
-// equal; with longer K the cut product wins.
+// stream and norm the result.  Its blocks own 16 columns and all of K, so the chip must hold them in
+// one round, and a CU pulls a block's weight rows at a limited rate, so K must be short or the
+// blocks must be nearly one a CU.  Measured in replayed graphs against the product cut along K over
+// blocks plus the norm kernel (us): 4096 x 4096 10.3 against 13.8 at 1 row, 12.1 against 14.5 at
+// 8, 13.0 against 14.8 at 16; 1024 x 3072 7.6 against 9.2 at 1 row, 9.4 against 9.7 at 16;
+// 4096 x 12288 22.8 against 25.6 at 2 rows, 25.3 against 26.6 at 8, 27.9 against 27.3 at 12 (every
+// block reads all activations, which is what more rows cost); 2560 x 9728 (160 blocks) 18.4 against
+// 17.4 and 5120 x 5120 (320 blocks, more than a round) 19.2 against 17.9 at 1 row: not taken.
 ROCML_EXPORT int rocml_gemm_residual_prescale_pays(int m, int n, int k) {
     if (m < 1 || m > 16 || k % 8 != 0) return 0;
     int tiles = ceil_div(n, 16);
-    const int cus = cu_count();       // a block a CU, or two
-    if (tiles <= cus && k <= 4096) return 1;
-    if (m <= 2 && tiles <= cus && k <= 12288) return 1;
-    if (m <= 2 && tiles <= 2 * cus && k <= 5120) return 1;
-    return 0;
+    const int cus = cu_count();
+    if (tiles > cus) return 0;
+    if (k <= 4096) return 1;
+    return k <= 12288 && m <= 8 && 10 * tiles >= 9 * cus;
 }
 
 // algo: 0 = choose, 1 = plain tiled kernel, 2 = MFMA tile kernel, 3 = MFMA few-rows kernel (M <= 64),
