@@ -418,6 +418,21 @@ FUSED_DECODE_HEAD_DIMS = (64, 128, 192, 256)
 FUSED_DECODE_PAGE = 64
 
 
+def decode_splits(pairs: int, n_cus: int, most: int) -> int:
+    """Splits of the key range for ``pairs`` (token, kv head) pairs of a decode step: about two
+    blocks a CU, and where that leaves CUs with unequal numbers of blocks (24 sequences of 8 kv
+    heads: 384 blocks on 256 CUs), up to four a CU if a multiple of the CUs can be had (768)."""
+    def waste(s: int) -> float:
+        blocks = pairs * s
+        return -(-blocks // n_cus) * n_cus / blocks - 1.0
+    base = max(1, 2 * n_cus // pairs)
+    best = base
+    for s in range(base + 1, max(base, 4 * n_cus // pairs) + 1):
+        if waste(s) < waste(best) - 0.1:
+            best = s
+    return max(1, min(best, most))
+
+
 def attention_decode_fusable(dtype: torch.dtype, n_heads: int, n_kv_heads: int, head_dim: int, page: int,
                              rot_dim: Optional[int]) -> bool:
     """Whether ``attention_decode_fused`` takes this layer: bfloat16 cache in pages of 64, a head

@@ -100,8 +100,7 @@ class Attention(Mixer):
         the sequences' lengths, so a recorded step can be replayed as they grow."""
         if step.max_new != 1:
             return 0
-        blocks = step.n_tokens * self.spec.n_kv_heads
-        return max(1, min(2 * self.n_cus // blocks, cache.block_table.shape[1], 64))
+        return ops.decode_splits(step.n_tokens * self.spec.n_kv_heads, self.n_cus, min(cache.block_table.shape[1], 64))
 
     def forward(self, step, xn, x_accum, cache, owns_cache: bool) -> None:
         s = self.spec

@@ -98,3 +98,14 @@ def test_catalog_and_resolve(tmp_path):
     (tmp_path / "config.json").write_text("{not json")
     with pytest.raises(ConfigError, match="JSON"):
         Qwen3Config.from_json(str(tmp_path))
+
+
+def test_decode_splits_fill_the_chip_evenly():
+    """Key-range splits of a decode step: about two blocks a CU, more where that would leave CUs
+    with unequal numbers of blocks, never more than the pages there are."""
+    from rocml_amd.ops import decode_splits
+    assert [decode_splits(b * 8, 256, 64) for b in (1, 2, 4, 8, 16, 32, 64, 128)] == [64, 32, 16, 8, 4, 2, 1, 1]
+    assert decode_splits(24 * 8, 256, 64) == 4          # 768 blocks, not 384 on 256 CUs
+    assert decode_splits(48 * 8, 256, 64) == 2
+    assert decode_splits(20 * 8, 256, 64) == 3          # 480 of 512 is near enough
+    assert decode_splits(8, 256, 5) == 5 and decode_splits(4096, 256, 64) == 1
