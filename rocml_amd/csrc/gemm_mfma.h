@@ -19,9 +19,14 @@
 //    workspace and are added in split order by a second kernel (or by the caller's next
 //    kernel), so results do not depend on timing
 //    (rocml-kernels/kernels/gemm_splitk_reduce.hip:4-10 has the same rule).
-//    gemm_skinny_ahead_kernel is the same for 17 to 64 rows, with weights and activations
-//    requested two steps ahead.
+//    gemm_skinny_ahead_kernel is the same with weights and activations requested two steps
+//    ahead and any number of waves a block from 2 to 16: for 17 to 64 rows, for the gated
+//    product at every number of rows up to 64 (it cannot be cut along K, so the waves a block
+//    are what makes its blocks one round over the CUs), and for products cut along K whose
+//    blocks the host chose for the busiest CU.
 //  * gemm_kpar_kernel, one or two rows: the waves of a block split K and meet once in LDS.
+//  * gemm_residual_prescale_kernel, up to 16 rows: whole sums into the residual stream and the
+//    next norm's operand in one pass.
 #pragma once
 #include "common.h"
 
