@@ -99,7 +99,7 @@ static int launch_mfma_tile(const void* x, int ldx, const void* w, int ldw, void
     return launch_mfma_tile_as<EPI, GemmTile128>(x, ldx, w, ldw, out, ldo, m, n, k, splits, workspace, plan, stream);
 }
 
-// The kernel for 17 to 64 rows on a product that cannot be cut along K (the gated product), with
+// The two-steps-ahead kernel on a product that cannot be cut along K (the gated product), with
 // WAVES waves a block, each on 16 columns.
 template <int MT, int EPI, int WAVES>
 static int launch_ahead_whole(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m, int n,
@@ -186,6 +186,13 @@ static double block_cost(BlockChoice c, int m, int row_tiles, int n, int cus) {
 
 static BlockChoice choose_blocks(BlockChoice usual, int m, int row_tiles, int n, int k, int cus,
                                  long long workspace_bytes, int skip_from, int skip_to) {
+    // (a step asks for the same few products over and over: the last answers are kept)
+    struct Kept { int m, row_tiles, n, k, cus; long long workspace_bytes; BlockChoice choice; bool set; };
+    static thread_local Kept kept[64];
+    Kept& slot = kept[((unsigned)n * 31u + (unsigned)k * 7u + (unsigned)m) % 64u];
+    if (slot.set && slot.m == m && slot.row_tiles == row_tiles && slot.n == n && slot.k == k && slot.cus == cus &&
+        slot.workspace_bytes == workspace_bytes)
+        return slot.choice;
     BlockChoice best = usual;
     double best_cost = 1e30;
     for (int kps = GS_KC; kps < k + GS_KC; kps += GS_KC) {
@@ -204,7 +211,9 @@ static BlockChoice choose_blocks(BlockChoice usual, int m, int row_tiles, int n,
     }
     // the usual blocks (four or eight waves, about two blocks or one a CU) unless the estimate
     // promises a clear gain: it is rough, and they are what the kernels were tuned with
-    return best_cost < 0.93 * block_cost(usual, m, row_tiles, n, cus) ? best : usual;
+    BlockChoice choice = best_cost < 0.93 * block_cost(usual, m, row_tiles, n, cus) ? best : usual;
+    slot = Kept{m, row_tiles, n, k, cus, workspace_bytes, choice, true};
+    return choice;
 }
 
 template <int MT, int EPI>
