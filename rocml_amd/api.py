@@ -128,11 +128,12 @@ class Model:
     def generate(self, prompts: Sequence[Sequence[int]],
                  sampling: Union[SamplingParams, Sequence[SamplingParams], None] = None,
                  max_new_tokens: int = 64, stop_tokens: Iterable[int] = (), ignore_eos: bool = False,
-                 on_step=None) -> List[Result]:
+                 on_step=None, on_token=None) -> List[Result]:
         """Continues every prompt (lists of token ids).  ``sampling`` is one set of parameters
         for all prompts or one per prompt; ``None`` means greedy.  A stop token ends its
         sequence and is not part of the result; the model's end-of-sequence ids are stop tokens
-        unless ``ignore_eos``.  ``on_step`` is called after every decode step with their number."""
+        unless ``ignore_eos``.  ``on_step`` is called after every decode step with their number,
+        ``on_token(prompt index, token id)`` for every token as it is drawn."""
         if sampling is None:
             sampling = SamplingParams.greedy()
         if isinstance(sampling, SamplingParams):
@@ -145,6 +146,7 @@ class Model:
         requests = [Request(list(p), max_new_tokens, s, stop) for p, s in zip(prompts, sampling)]
         gen = Generator(EngineBackend(self.engine), max_batch=self.options.max_batch)
         gen.on_step = on_step
+        gen.on_token = on_token
         results = gen.run(requests)
         self.last_stats = gen.stats
         return results

@@ -76,16 +76,40 @@ def cmd_generate(args) -> int:
     params = sampling_from_args(args, model.entry.sampling if model.entry else None)
     profiler = _profiler(args.dtype) if args.profile else None
     kwargs = dict(max_new_tokens=args.n, stop_tokens=_parse_ids(args.stop_ids or ""), ignore_eos=args.ignore_eos)
+    # One prompt is written out as it is generated, token by token
+    # (rocml-cli/src/cmd_generate.rs:113-127); several are written when all are done.
+    streamed = len(prompts) == 1
+    if streamed:
+        shown = []
+
+        def on_token(_index: int, token: int) -> None:
+            if tok is not None:
+                shown.append(token)
+                text = tok.decode(shown)
+                if not text.endswith("\ufffd"):            # (a piece may end inside a character)
+                    sys.stdout.write(text[on_token.written:])
+                    on_token.written = len(text)
+            else:
+                sys.stdout.write(("" if on_token.written == 0 else " ") + str(token))
+                on_token.written += 1
+            sys.stdout.flush()
+        on_token.written = 0
+        kwargs["on_token"] = on_token
     if profiler is not None:
         with profiler:
             results = model.generate(prompts, params, **kwargs)
     else:
         results = model.generate(prompts, params, **kwargs)
-    for i, r in enumerate(results):
-        if tok is not None and i == len(results) - 1 and args.prompt is not None:
-            print(tok.decode(r.tokens))
-        else:
-            print(" ".join(str(t) for t in r.tokens))
+    if streamed:
+        if tok is not None:
+            sys.stdout.write(tok.decode(results[0].tokens)[on_token.written:])    # what a held-back piece left
+        print()
+    else:
+        for i, r in enumerate(results):
+            if tok is not None and i == len(results) - 1 and args.prompt is not None:
+                print(tok.decode(r.tokens))
+            else:
+                print(" ".join(str(t) for t in r.tokens))
     s = model.last_stats
     print(f"prompt: {s.prompt_tokens} tokens in {s.prompt_seconds:.3f} s ({s.prompt_tok_s():.1f} tok/s); "
           f"generated: {s.generated_tokens} tokens in {s.decode_seconds:.3f} s ({s.decode_tok_s():.1f} tok/s)",

@@ -159,6 +159,10 @@ class Generator:
         # called with the number of decode steps run so far after each of them: a place for a
         # benchmark to take its times without a loop of its own
         self.on_step = None
+        # called as on_token(request index, token id) for every token as it is drawn, in the order
+        # of the batch (the reference hands every piece to a callback as it is decoded,
+        # rocml/src/generate/mod.rs:67-85)
+        self.on_token = None
 
     def _final_length(self, r: Request) -> int:
         return min(len(r.prompt) + r.max_new_tokens, self.backend.max_positions)
@@ -249,6 +253,8 @@ class Generator:
                     s.out.append(tok)
                     s.sampling.history.append(tok)
                     self.stats.generated_tokens += 1
+                    if self.on_token is not None:
+                        self.on_token(s.index, tok)
                     if len(s.out) >= s.request.max_new_tokens:
                         reason = "length"
                     elif len(s.request.prompt) + len(s.out) >= be.max_positions:

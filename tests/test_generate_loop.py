@@ -88,6 +88,23 @@ def test_stop_token_is_not_emitted_and_frees_the_slot():
     assert all(0 in s for s in be.steps[:gone]) and all(0 not in s for s in be.steps[gone:])
 
 
+def test_every_token_is_handed_out_as_it_is_drawn():
+    """``on_token`` sees every emitted token of every request once, in the order they were drawn
+    (a step's tokens in the order of the batch), and never a stop token."""
+    full, _ = _expected([5, 6], 10)
+    stop = full[3]
+    reqs = [Request([5, 6], 10, stop_tokens=frozenset([stop])), Request([1], 4), Request([], 3), Request([2, 2], 6)]
+    seen = []
+    gen = Generator(Scripted(slots=2), max_batch=2)
+    gen.on_token = lambda index, token: seen.append((index, token))
+    res = gen.run(reqs)
+    for i, r in enumerate(res):
+        assert [t for j, t in seen if j == i] == r.tokens
+    assert stop not in [t for j, t in seen if j == 0] and len(seen) == sum(len(r.tokens) for r in res)
+    firsts = [j for j, _ in seen[:2]]
+    assert firsts == [0, 1]                       # the first step's tokens in the order of the batch
+
+
 def test_batches_follow_slots_and_room_and_reuse_slots():
     be = Scripted(slots=2)
     reqs = [Request([i + 1], 3) for i in range(5)]
