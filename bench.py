@@ -97,7 +97,10 @@ def main() -> int:
         def step(self, slots, tokens):
             if all(len(t) == 1 for t in tokens):
                 return super().step(slots, tokens)
-            self.engine.adopt_positions(slots, [len(t) for t in tokens])
+            cache = self.engine.cache
+            new_lens = [cache.length(s) + len(t) for s, t in zip(slots, tokens)]
+            cache.reserve(list(slots), new_lens)
+            cache.commit(list(slots), new_lens)
             return torch.zeros((len(slots), spec.vocab), dtype=torch.float32, device=model.device)
 
     def decode(batch: int, steps: int, warmup: int):

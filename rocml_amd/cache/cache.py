@@ -273,9 +273,11 @@ def register_cache_group(request_type: type, group_type: type) -> None:
 
 
 def _group_type(req) -> type:
-    for rt, gt in _GROUP_KINDS.items():
-        if isinstance(req, rt):
-            return gt
+    # the request's own class first, then its bases from the nearest on: a request class that
+    # derives from a registered one and registers a group of its own gets that group
+    for rt in type(req).__mro__:
+        if rt in _GROUP_KINDS:
+            return _GROUP_KINDS[rt]
     raise RocmlError(f"unknown cache request {req!r}")
 
 

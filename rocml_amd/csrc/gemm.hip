@@ -187,11 +187,15 @@ static double block_cost(BlockChoice c, int m, int row_tiles, int n, int cus) {
 static BlockChoice choose_blocks(BlockChoice usual, int m, int row_tiles, int n, int k, int cus,
                                  long long workspace_bytes, int skip_from, int skip_to) {
     // (a step asks for the same few products over and over: the last answers are kept)
-    struct Kept { int m, row_tiles, n, k, cus; long long workspace_bytes; BlockChoice choice; bool set; };
+    // (the answer depends on the usual blocks and on the skipped wave counts too, which differ
+    // between the callers that share this table)
+    struct Kept { int m, row_tiles, n, k, cus; long long workspace_bytes; BlockChoice usual; int skip_from, skip_to;
+                  BlockChoice choice; bool set; };
     static thread_local Kept kept[64];
     Kept& slot = kept[((unsigned)n * 31u + (unsigned)k * 7u + (unsigned)m) % 64u];
     if (slot.set && slot.m == m && slot.row_tiles == row_tiles && slot.n == n && slot.k == k && slot.cus == cus &&
-        slot.workspace_bytes == workspace_bytes)
+        slot.workspace_bytes == workspace_bytes && slot.usual.waves == usual.waves && slot.usual.splits == usual.splits &&
+        slot.usual.k_per_split == usual.k_per_split && slot.skip_from == skip_from && slot.skip_to == skip_to)
         return slot.choice;
     BlockChoice best = usual;
     double best_cost = 1e30;
@@ -212,7 +216,7 @@ static BlockChoice choose_blocks(BlockChoice usual, int m, int row_tiles, int n,
     // the usual blocks (four or eight waves, about two blocks or one a CU) unless the estimate
     // promises a clear gain: it is rough, and they are what the kernels were tuned with
     BlockChoice choice = best_cost < 0.93 * block_cost(usual, m, row_tiles, n, cus) ? best : usual;
-    slot = Kept{m, row_tiles, n, k, cus, workspace_bytes, choice, true};
+    slot = Kept{m, row_tiles, n, k, cus, workspace_bytes, usual, skip_from, skip_to, choice, true};
     return choice;
 }
 

@@ -2,10 +2,9 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-// rocml_argmax_static has no counterpart in the reference (which picks the greedy token on the
-// host, rocml/src/sample.rs:172-182).  It is rocml_argmax for callers that cannot allocate device
-// memory or carry a workspace around: code under HIP graph capture, tight serving loops, harnesses
-// that forbid hipMalloc.  The partial results of its two stages live in an array of the library
+// rocml_argmax_static has no counterpart in the reference.  It is rocml_argmax for callers that
+// cannot allocate device memory or carry a workspace around: code under HIP graph capture, tight
+// serving loops, harnesses that forbid hipMalloc.  The partial results of its two stages live in an array of the library
 // itself, ROCML_ARGMAX_STATIC_MAX_ROWS * 64 32-bit words (256 KiB) that every GPU the library
 // runs on holds until the process ends; the call allocates and frees nothing.
 //

@@ -58,17 +58,6 @@ class Engine:
     def length(self, slot: int) -> int:
         return self.cache.length(slot)
 
-    def adopt_positions(self, slots: Sequence[int], counts: Sequence[int]) -> None:
-        """Lengthens sequences by ``counts`` positions without running tokens: the cache rows are
-        whatever the pages held.  For measurements that want decode steps at a given depth
-        without paying for the prompt; results of such sequences mean nothing."""
-        new_lens = [self.cache.length(s) + n for s, n in zip(slots, counts)]
-        if max(new_lens) > self.model.spec.max_positions:
-            raise ContextOverflowError(f"a sequence would reach {max(new_lens)} positions; the model has "
-                                       f"{self.model.spec.max_positions}")
-        self.cache.reserve(list(slots), new_lens)
-        self.cache.commit(list(slots), new_lens)
-
     # -- the step ------------------------------------------------------------------------
     def step(self, entries: Sequence[StepEntry], device_ids: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Runs the entries' tokens; returns ``[n_wanted, vocab]`` 32-bit logits on the
@@ -113,7 +102,10 @@ class Engine:
         # The step as pieces of at most max_step_tokens tokens (a sequence may straddle pieces).
         # Pages are reserved piece by piece, and a piece is committed before the next runs, so a
         # group with a window gives pages back while a long prompt passes through it; the whole
-        # plan is checked against the free pages first, so a step runs entirely or not at all.
+        # plan is checked against the free pages first, so a step is never left half run for want
+        # of pages.  (Any other failure inside a piece, a kernel's refusal say, leaves the pieces
+        # before it committed: the caller then releases the step's sequences, as the generation
+        # loop does.)
         total = sum(counts)
         n_want_total = sum(len(e.want) for e in entries)
         pieces = None
@@ -147,7 +139,9 @@ class Engine:
                 p_dest.extend(int(want_base[i]) + k for k, _ in wanted)
             p_lens = [s + len(t) for s, t in zip(p_starts, p_tokens)]
             self.cache.reserve(p_slots, p_lens, which="windowed")
-            logits = self._run_piece(p_slots, p_starts, p_tokens, p_want)
+            # (ids on the device come one per entry, so a piece's entries are a run of them)
+            p_ids = None if device_ids is None else device_ids[piece[0][0]:piece[0][0] + len(piece)]
+            logits = self._run_piece(p_slots, p_starts, p_tokens, p_want, p_ids)
             if logits is not None:
                 result[torch.as_tensor(p_dest, device=self.model.device)] = logits
             self.cache.commit(p_slots, p_lens)

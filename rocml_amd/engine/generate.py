@@ -70,7 +70,7 @@ class EngineBackend:
         self.max_positions = engine.model.spec.max_positions
         self.run_ahead = run_ahead and hasattr(self.sampler, "sample_start")
         self._row_slots: Optional[List[int]] = None     # the slots whose logits the last step returned, row by row
-        self._ahead = None                              # (slots, logits, slots still live) of a step launched ahead
+        self._ahead = None                              # (slots, logits, slots still live, ids drawn) of a step launched ahead
 
     def can_admit(self, lengths: Sequence[int], prompts: Optional[Sequence[int]] = None) -> bool:
         """Whether new sequences with prompts of ``prompts`` tokens that will grow to ``lengths``
@@ -96,8 +96,18 @@ class EngineBackend:
         from .batch import StepEntry
         slots = list(slots)
         ahead, self._ahead = self._ahead, None
-        if ahead is not None and all(len(t) == 1 for t in tokens) and set(slots) <= ahead[2]:
-            # the step is running already (with these tokens: they are what the sampler drew)
+        covered = set() if ahead is None else set(slots) & ahead[2]
+        if covered and (len(covered) != len(slots) or any(len(t) != 1 for t in tokens)):
+            # some of these sequences are one token further already: running them again would
+            # advance them twice
+            raise RocmlError("a step was launched ahead for sequences %s; the next step must continue them all "
+                             "with the one token each that was drawn" % sorted(covered))
+        if covered:
+            # the step is running already, with the tokens the sampler drew
+            drawn = ahead[3]
+            for s, t in zip(slots, tokens):
+                if s in drawn and int(t[0]) != drawn[s]:
+                    raise RocmlError(f"sequence {s} was run ahead with token {drawn[s]}, not {int(t[0])}")
             self._row_slots = slots
             if slots == ahead[0]:
                 return ahead[1]
@@ -126,10 +136,13 @@ class EngineBackend:
                 # those sequences one token further, as if none of them drew a stop token; refused (a
                 # full cache) it changes nothing and the loop goes on step by step
                 ahead = self.engine.step([StepEntry(s, [0], [0]) for s in slots], device_ids=ids)
-                self._ahead = (slots, ahead, set(slots))
+                self._ahead = (slots, ahead, set(slots), {})
             except RocmlError:
                 self._ahead = None
-        return self.sampler.finish(started)
+        drawn = self.sampler.finish(started)
+        if self._ahead is not None:
+            self._ahead[3].update((self._row_slots[b], int(drawn[b])) for b in rows)
+        return drawn
 
     def synchronize(self) -> None:
         import torch

@@ -46,17 +46,15 @@ def rope_neox(x: torch.Tensor, positions: Sequence[int], theta: float) -> torch.
     position (rocml/src/forward/attention.rs:125-140)."""
     tokens, heads, d = x.shape
     half = d // 2
+    # angles in float64 whatever the type of x: a = pos * theta^(-2i/D), one row per token
+    inv_freq = torch.tensor([theta ** (-2.0 * i / d) for i in range(half)], dtype=torch.float64)
+    angle = torch.tensor([float(p) for p in positions], dtype=torch.float64)[:, None] * inv_freq[None, :]
+    c = torch.cos(angle).to(x.dtype)[:, None, :]
+    s = torch.sin(angle).to(x.dtype)[:, None, :]
+    x0, x1 = x[:, :, :half], x[:, :, half:2 * half]
     out = x.clone()
-    for t in range(tokens):
-        pos = float(positions[t])
-        for i in range(half):
-            inv_freq = theta ** (-2.0 * i / d)
-            a = pos * inv_freq
-            c, s = math.cos(a), math.sin(a)
-            x0 = x[t, :, i]
-            x1 = x[t, :, i + half]
-            out[t, :, i] = x0 * c - x1 * s
-            out[t, :, i + half] = x0 * s + x1 * c
+    out[:, :, :half] = x0 * c - x1 * s
+    out[:, :, half:2 * half] = x0 * s + x1 * c
     return out
 
 
@@ -88,13 +86,16 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     hkv = k.shape[1]
     group = hq // hkv
     out = torch.zeros_like(q)
+    place = torch.arange(t_len)
+    seen = place[None, :] <= place[:, None]                  # row p sees columns j <= p
+    if window is not None:
+        seen &= place[None, :] > place[:, None] - window     # ... and j >= p - window + 1
     for h in range(hq):
         kv = h // group
-        for p in range(t_len):
-            lo = 0 if window is None else max(0, p - window + 1)
-            scores = (k[lo:p + 1, kv] @ q[p, h]) * scale
-            e = torch.exp(scores - scores.max())
-            out[p, h] = (rounded(e) @ v[lo:p + 1, kv]) / e.sum()
+        scores = (q[:, h] @ k[:, kv].T) * scale
+        scores = scores.masked_fill(~seen, float("-inf"))
+        e = torch.exp(scores - scores.max(dim=-1, keepdim=True).values)   # 0 where a key is not seen
+        out[:, h] = (rounded(e) @ v[:, kv]) / e.sum(dim=-1, keepdim=True)
     return out
 
 

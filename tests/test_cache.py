@@ -267,3 +267,28 @@ def test_a_cache_group_kind_of_its_own_needs_no_change_to_the_cache():
     c.free_sequence(a)
     c.check()
     assert latent.tokens_seen == {b: 5} and c.line(2)[0] is latent and c.line(2)[1] == 1
+
+
+def test_a_request_class_derived_from_a_registered_one_gets_its_own_group():
+    """The nearest registered class of a request decides: a subclass of the key/value request that
+    registers a group of its own is served by that group, an unregistered subclass by its base's."""
+    from dataclasses import dataclass
+    from rocml_amd.cache import register_cache_group
+    from rocml_amd.cache.cache import KVGroup, _group_type
+
+    @dataclass(frozen=True)
+    class WideRequest(KVCacheRequest):
+        pass
+
+    @dataclass(frozen=True)
+    class PlainChild(KVCacheRequest):
+        pass
+
+    class WideGroup(KVGroup):
+        pass
+
+    register_cache_group(WideRequest, WideGroup)
+    assert _group_type(WideRequest(1, 16)) is WideGroup
+    assert _group_type(PlainChild(1, 16)) is KVGroup and _group_type(KVCacheRequest(1, 16)) is KVGroup
+    c = Cache([WideRequest(1, 16), KVCacheRequest(1, 16)], max_tokens=128, dtype=torch.float32, device="cpu")
+    assert type(c.line(0)[0]) is WideGroup and type(c.line(1)[0]) is KVGroup

@@ -293,3 +293,41 @@ def test_running_ahead_stops_at_the_models_last_position():
     want = Generator(Scripted(max_positions=6), max_batch=2).run([Request([1, 2, 3], 10), Request([4], 3)])
     assert [(r.tokens, r.finish_reason) for r in got] == [(r.tokens, r.finish_reason) for r in want]
     assert got[0].finish_reason == "context" and all(len(h) <= 6 for h in engine.history.values())
+
+
+def test_a_step_that_does_not_continue_the_one_launched_ahead_is_refused():
+    """After sampling with run-ahead the sequences are one token further already: a next step for
+    only some of them with others beside, or with another token than the one drawn, would advance
+    them twice or feed them something they were not run with; the backend says so."""
+    import torch
+    from rocml_amd.engine.generate import EngineBackend
+    from rocml_amd.sampling import SamplingParams
+    from rocml_amd.sampling.sampler import SequenceSampling
+
+    def start():
+        engine = _FakeEngine(slots=3)
+        backend = EngineBackend(engine, sampler=_FakeSampler())
+        slots = [backend.new_sequence() for _ in range(3)]
+        logits = backend.step(slots[:2], [[1, 2], [3]])
+        seqs = [SequenceSampling(SamplingParams.greedy(), None, []) for _ in range(2)]
+        drawn = backend.sample(logits, seqs, [True, True])
+        return backend, slots, drawn
+
+    backend, slots, drawn = start()
+    assert backend.step(slots[:2], [[drawn[0]], [drawn[1]]]).shape[0] == 2        # the step that was launched
+    backend, slots, drawn = start()
+    assert backend.step(slots[1:2], [[drawn[1]]]).shape[0] == 1                   # a subset: its rows are picked
+    backend, slots, drawn = start()
+    with pytest.raises(RocmlError, match="launched ahead"):
+        backend.step(slots[1:3], [[drawn[1]], [5]])                                # one ran ahead, one did not
+    backend, slots, drawn = start()
+    with pytest.raises(RocmlError, match="run ahead with token"):
+        backend.step(slots[:2], [[drawn[0]], [drawn[1] + 1]])
+    backend, slots, drawn = start()
+    with pytest.raises(RocmlError, match="launched ahead"):
+        backend.step(slots[:1], [[drawn[0], 4]])                                   # more than the one token
+    backend, slots, drawn = start()
+    backend.release(slots[0])
+    backend.release(slots[1])
+    s = backend.new_sequence()                                                      # a slot that ran ahead, now another sequence
+    assert backend.step([s], [[1, 2, 3]]).shape[0] == 1

@@ -335,3 +335,64 @@ def test_refusals():
     dev, *_ = _build([(10, 1)], 4, 3, 32, torch.bfloat16, 0)
     with pytest.raises(KernelError):
         _run(dev, [(10, 1)], 4, 3, 32, 1.0, None, PLAIN)     # 4 heads over 3 kv heads
+
+
+# ---- contexts of tens of thousands of tokens ---------------------------------------------------
+def _reference_rows(q, k, v, positions, scale, window):
+    """The same as ``_reference`` without loops over positions: q [n, Hq, D] at ``positions``,
+    k, v [L, Hkv, D], everything in float64, a head at a time."""
+    n, hq, d = q.shape
+    group = hq // k.shape[1]
+    pos = torch.tensor(positions)
+    keys = torch.arange(k.shape[0])
+    seen = keys[None, :] <= pos[:, None]
+    if window is not None:
+        seen &= keys[None, :] > pos[:, None] - window
+    out = torch.zeros(n, hq, d, dtype=torch.float64)
+    for h in range(hq):
+        s = (q[:, h].double() @ k[:, h // group].double().T) * scale
+        s = s.masked_fill(~seen, float("-inf"))
+        out[:, h] = torch.softmax(s, dim=-1) @ v[:, h // group].double()
+    return out
+
+
+def _needles(length, n_new):
+    """Places whose keys are made to carry the weight: the ends of the sequence, both sides of
+    page borders near and far, the middle."""
+    first_new = length - n_new
+    places = {0, 63, 64, 4095, 4096, length // 2 + 17, first_new - 65, first_new - 64, first_new - 1, first_new - 4000}
+    return sorted(p for p in places if 0 <= p < first_new)
+
+
+def _long_case(length, n_new, hq, hkv, d, window, n_splits, seed):
+    """A sequence of ``length`` positions whose last ``n_new`` are the step's: among the random
+    keys a handful point along the first query of their kv head, four times as long, so that
+    those few share nearly all weight and each of them missing, doubled or taken from a wrong
+    page moves the output by a tenth and more."""
+    seqs = [(length, n_new)]
+    dev, ks, vs, qs = _build(seqs, hq, hkv, d, torch.bfloat16, seed, spare_pages=5)
+    group = hq // hkv
+    k, table = ks[0], dev["table"].cpu()
+    for j in range(hkv):
+        lead = qs[0][0, j * group].float()
+        for p in _needles(length, n_new):
+            k[p, j] = (4.0 * lead).to(torch.bfloat16)
+            dev["kc"][int(table[0, p // PAGE]), j, p % PAGE] = k[p, j].cuda()
+    scale = 1.0 / math.sqrt(d)
+    got = _run(dev, seqs, hq, hkv, d, scale, window, MFMA, n_splits).double().reshape(-1, hq, d)
+    ref = _reference_rows(qs[0], k, vs[0], list(range(length - n_new, length)), scale, window)
+    err = float((got - ref).abs().max())
+    assert err < 1.5e-2, f"length {length}, {n_new} new, window {window}, {n_splits} splits: error {err}"
+    # (the needles do decide: without them the first head's output is another one)
+    assert float((ref[0, 0] - vs[0][:length - n_new, 0].double().mean(0)).abs().max()) > 0.1
+
+
+@pytest.mark.parametrize("length", [32768, 40960])
+@pytest.mark.parametrize("window,n_splits", [(None, 1), (None, 8), (None, 64), (None, 0), (4096, 8), (4096, 64), (70, 0)])
+def test_decode_over_tens_of_thousands_of_keys(length, window, n_splits):
+    _long_case(length, 1, 8, 2, 128, window, n_splits, seed=31)
+
+
+@pytest.mark.parametrize("length,window", [(32768, None), (32768, 5000), (40960, None)])
+def test_a_chunk_deep_in_a_long_sequence(length, window):
+    _long_case(length, 256, 4, 2, 128, window, 0, seed=32)

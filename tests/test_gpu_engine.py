@@ -39,6 +39,19 @@ def _oracle_weights(weights, dtype):
     return {k: (v if v.dim() == 1 else v.to(torch.bfloat16).to(torch.float32)) for k, v in weights.items()}
 
 
+# The worst position's largest difference over that position's largest logit: 32-bit against the
+# plain implementation, bfloat16 against the plain implementation rounding where the engine does.
+POSITION_TOL = 1e-4
+ROUNDED_TOL = 1e-2
+
+
+def _rounding_oracle(cfg, weights, p, few_tokens=False):
+    plain_kernel = cfg["head_dim"] not in (32, 64, 96, 128, 192, 256)
+    return plain.forward(cfg, weights, p, rounded=plain.round_bfloat16,
+                         rounded_probs=(lambda t: t) if plain_kernel else None,
+                         ffn_norm_rounds_before_scale=few_tokens and cfg["hidden_size"] % 8 == 0)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F", "G", "H"])
 def test_whole_tail_and_batches(models, name, dtype):
@@ -48,18 +61,26 @@ def test_whole_tail_and_batches(models, name, dtype):
     prompts = [helpers.random_tokens(n, cfg["vocab_size"], 100 + i) for i, n in enumerate(LENGTHS[name])]
     refs = [plain.forward(cfg, oracle_w, p) for p in prompts]
     tol = TOL[dtype]
-    for p, ref in zip(prompts, refs):
-        got = helpers.run_whole(engine, p)
-        assert helpers.rel_to_max(got, ref) < tol, f"whole, length {len(p)}"
-        got = helpers.run_tail_by_one(engine, p, 32)
-        assert helpers.rel_to_max(got, ref) < tol, f"tail by one, length {len(p)}"
+    # Position by position as well, so that one bad place does not hide under the largest logit of
+    # a whole request: in bfloat16 against the oracle that rounds where the engine does.
+    sharp_refs, sharp_tol = refs, POSITION_TOL
+    if dtype == "bfloat16":
+        sharp_refs, sharp_tol = [_rounding_oracle(cfg, weights, p) for p in prompts], ROUNDED_TOL
+
+    def check(got, i, what):
+        assert helpers.rel_to_max(got, refs[i]) < tol, what
+        assert helpers.per_position(got, sharp_refs[i]) < sharp_tol, what + " (position by position)"
+
+    for i, p in enumerate(prompts):
+        check(helpers.run_whole(engine, p), i, f"whole, length {len(p)}")
+        check(helpers.run_tail_by_one(engine, p, 32), i, f"tail by one, length {len(p)}")
     # Two batches one after the other: the second uses the slots and pages of the first.
     for order in (list(range(len(prompts))), list(reversed(range(len(prompts))))):
         batch = [prompts[i] for i in order]
         n_prefill = [max(1, len(p) - 3 * (j + 1)) for j, p in enumerate(batch)]
         got = helpers.run_batch(engine, batch, n_prefill)
         for j, i in enumerate(order):
-            assert helpers.rel_to_max(got[j], refs[i]) < tol, f"batch order {order}, sequence {i}"
+            check(got[j], i, f"batch order {order}, sequence {i}")
     engine.cache.check()
     assert not engine.cache.lengths
 
@@ -141,7 +162,6 @@ def test_refused_steps_leave_the_engine_as_it_was(models):
 # relative to the largest score seen so far, which in a decode step (cached keys, then the new
 # one) is not the largest of all, and only the loose bound holds there.
 ALIKE_TOL = 1e-5
-ROUNDED_TOL = 1e-2
 
 
 @pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "G", "H"])
@@ -151,9 +171,7 @@ def test_bfloat16_against_an_oracle_that_rounds_where_the_engine_does(models, na
     plain_kernel = cfg["head_dim"] not in (32, 64, 96, 128, 192, 256)
 
     def oracle(p, few_tokens=False):
-        return plain.forward(cfg, weights, p, rounded=plain.round_bfloat16,
-                             rounded_probs=(lambda t: t) if plain_kernel else None,
-                             ffn_norm_rounds_before_scale=few_tokens and cfg["hidden_size"] % 8 == 0)
+        return _rounding_oracle(cfg, weights, p, few_tokens)
     short = [helpers.random_tokens(2 + i % 4, cfg["vocab_size"], 400 + i) for i in range(12)]
     whole = [helpers.per_position(helpers.run_whole(engine, p), oracle(p, True)) for p in short]
     assert max(whole) < ROUNDED_TOL
@@ -173,9 +191,9 @@ def test_bfloat16_against_an_oracle_that_rounds_where_the_engine_does(models, na
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,n_seqs", [("H", 33), ("H", 64), ("F", 33), ("F", 64)])
+@pytest.mark.parametrize("name,n_seqs", [("H", 33), ("H", 64), ("F", 33), ("F", 64), ("H", 130), ("F", 100)])
 def test_many_sequences_in_a_step(models, name, dtype, n_seqs):
-    """33 and 64 sequences of unequal lengths: their prompts in one step, then decode steps in
+    """33 to 130 sequences of unequal lengths (beyond 64 rows every product is the tile kernel's): their prompts in one step, then decode steps in
     which the shorter requests end one after the other, so the batch shrinks through the row
     counts the few-rows kernels are built for; then the same slots again with every sequence
     decoding side by side, the steps recorded once and replayed.  H takes the decode attention
@@ -191,6 +209,11 @@ def test_many_sequences_in_a_step(models, name, dtype, n_seqs):
     got = helpers.run_batch(engine, seqs, lengths)
     worst = max(helpers.rel_to_max(g, r) for g, r in zip(got, refs))
     assert worst < TOL[dtype], f"{n_seqs} sequences: {worst}"
+    sharp_refs, sharp_tol = refs, POSITION_TOL
+    if dtype == "bfloat16":
+        sharp_refs, sharp_tol = [_rounding_oracle(cfg, weights, s) for s in seqs], ROUNDED_TOL
+    worst = max(helpers.per_position(g, r) for g, r in zip(got, sharp_refs))
+    assert worst < sharp_tol, f"{n_seqs} sequences, position by position: {worst}"
     engine.cache.check()
     assert not engine.cache.lengths
     slots = [engine.new_sequence() for _ in seqs]
@@ -199,6 +222,7 @@ def test_many_sequences_in_a_step(models, name, dtype, n_seqs):
         logits = engine.step([StepEntry(s, [q[k]], [0]) for s, q in zip(slots, seqs)]).cpu()
         expect = torch.stack([r[k] for r in refs])
         assert helpers.rel_to_max(logits, expect) < TOL[dtype], f"decode step {k}"
+        assert helpers.per_position(logits, torch.stack([r[k] for r in sharp_refs])) < sharp_tol, f"decode step {k}, row by row"
     recorded = [key for key, entry in engine._graphs.items() if entry[1] is not None]
     assert engine.use_graphs and any(key[0] == n_seqs for key in recorded)
     for s in slots:

@@ -262,3 +262,20 @@ def test_a_catalog_model_has_the_weights_its_written_folder_has(tmp_path):
     assert [r.tokens for r in by_name.generate(prompts, max_new_tokens=6)] == \
         [r.tokens for r in from_folder.generate(prompts, max_new_tokens=6)]
     assert not torch.equal(Model.load("tiny-b", dtype="float32", seed=6, ctx=64).engine.model.embed, a.embed)
+
+
+def test_a_decode_step_cut_into_pieces_runs_the_ids_that_were_drawn(models):
+    """With fewer tokens to a step than the batch has sequences every decode step runs in pieces;
+    a step launched ahead of the host takes its ids from the sampler's output on the device, and
+    every piece must take its own run of them."""
+    from rocml_amd.engine import Engine, EngineBackend, Generator, Request
+    from rocml_amd.weights import load_model
+    path, cfg, weights = models["B"]
+    prompts = [helpers.random_tokens(n, cfg["vocab_size"], 140 + i) for i, n in enumerate([4, 1, 9, 2, 6, 3, 5])]
+    want = [plain.greedy(cfg, weights, p, 6) for p in prompts]
+    for run_ahead in (True, False):
+        engine = Engine(load_model(path, dtype="float32", device="cuda:0"), max_tokens=7 * 64, max_seqs=7, max_step_tokens=3)
+        reqs = [Request(list(p), 6) for p in prompts]
+        got = Generator(EngineBackend(engine, run_ahead=run_ahead), max_batch=7).run(reqs)
+        assert [r.tokens for r in got] == want, f"run_ahead={run_ahead}"
+        engine.cache.check()
