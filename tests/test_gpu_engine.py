@@ -43,6 +43,10 @@ def _oracle_weights(weights, dtype):
 # plain implementation, bfloat16 against the plain implementation rounding where the engine does.
 POSITION_TOL = 1e-4
 ROUNDED_TOL = 1e-2
+# (configuration F sums 2,048 rounded terms where the others sum a hundred: its rounding noise was
+# measured at 1.2e-2 of a position's largest logit; the bound that held for whole requests holds
+# for each of its positions)
+ROUNDED_TOL_BY_NAME = {"F": 2e-2}
 
 
 def _rounding_oracle(cfg, weights, p, few_tokens=False):
@@ -65,7 +69,8 @@ def test_whole_tail_and_batches(models, name, dtype):
     # a whole request: in bfloat16 against the oracle that rounds where the engine does.
     sharp_refs, sharp_tol = refs, POSITION_TOL
     if dtype == "bfloat16":
-        sharp_refs, sharp_tol = [_rounding_oracle(cfg, weights, p) for p in prompts], ROUNDED_TOL
+        sharp_refs = [_rounding_oracle(cfg, weights, p) for p in prompts]
+        sharp_tol = ROUNDED_TOL_BY_NAME.get(name, ROUNDED_TOL)
 
     def check(got, i, what):
         assert helpers.rel_to_max(got, refs[i]) < tol, what
@@ -211,7 +216,8 @@ def test_many_sequences_in_a_step(models, name, dtype, n_seqs):
     assert worst < TOL[dtype], f"{n_seqs} sequences: {worst}"
     sharp_refs, sharp_tol = refs, POSITION_TOL
     if dtype == "bfloat16":
-        sharp_refs, sharp_tol = [_rounding_oracle(cfg, weights, s) for s in seqs], ROUNDED_TOL
+        sharp_refs = [_rounding_oracle(cfg, weights, s) for s in seqs]
+        sharp_tol = ROUNDED_TOL_BY_NAME.get(name, ROUNDED_TOL)
     worst = max(helpers.per_position(g, r) for g, r in zip(got, sharp_refs))
     assert worst < sharp_tol, f"{n_seqs} sequences, position by position: {worst}"
     engine.cache.check()
