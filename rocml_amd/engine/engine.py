@@ -46,6 +46,8 @@ class Engine:
         self.steps_run = 0
         self.use_graphs = use_graphs and model.graph_safe
         self.max_graph_batch = 256
+        self.max_graph_prompt_tokens = 1024     # prompt steps of at most so many tokens may be recorded
+        self.max_prompt_graphs = 32
         self._graphs: Dict[tuple, tuple] = {}
 
     # -- sequences -----------------------------------------------------------------------
@@ -206,19 +208,27 @@ class Engine:
 
         profile.set_phase("decode" if max_new == 1 else "prefill")
         # (a profiler times single launches: no recorded graph while one is active)
-        if not (self.use_graphs and max_new == 1 and len(slots) <= self.max_graph_batch) or profile.active() is not None:
+        if not self.use_graphs or len(slots) > self.max_graph_batch or profile.active() is not None:
             return run(context())
-        # Decode steps of one shape run from a recorded graph: the launches of a step are the
-        # same every time, only the integer tables change, and those lie at fixed addresses.
-        # A shape runs plainly the first time (kernels set themselves up, buffers reach their
-        # size), is recorded the second time, and replayed from then on.
-        key = (len(slots), n_want, width)
+        # Steps of one shape run from a recorded graph: the launches of a step are the same every
+        # time, only the integer tables change, and those lie at fixed addresses.  A decode step's
+        # shape is its number of sequences; a prompt step's is every sequence's number of tokens
+        # and first position (short prompts only: a long one keeps the GPU busy far longer than
+        # the host needs to launch it).  A shape runs plainly the first time (kernels set
+        # themselves up, buffers reach their size), is recorded the second time, and replayed
+        # from then on.
+        if max_new == 1:
+            key = (len(slots), n_want, width)
+        elif self.model.prompt_graph_safe and int(ids.size) <= self.max_graph_prompt_tokens:
+            key = ("prompt", tuple(len(t) for t in tokens), tuple(starts), n_want, width)
+        else:
+            return run(context())
         entry = self._graphs.get(key)
         if entry is not None and entry[0] != self.workspace.generation:
             entry = None                      # a buffer moved: the recorded addresses are stale
         if entry is None:
             result = run(context())
-            self._graphs[key] = (self.workspace.generation, None, None)
+            self._remember(key, (self.workspace.generation, None, None))
             return result
         generation, graph, result = entry
         if graph is None:
@@ -230,6 +240,15 @@ class Engine:
                 # recording allocated a buffer after all; run plainly and start over
                 del self._graphs[key]
                 return run(context())
-            self._graphs[key] = (generation, graph, result)
+            self._remember(key, (generation, graph, result))
         graph.replay()
         return result
+
+    def _remember(self, key, entry) -> None:
+        """Keeps a shape's graph; of the prompt shapes only the ``max_prompt_graphs`` seen last."""
+        self._graphs.pop(key, None)
+        self._graphs[key] = entry                      # (a dict keeps insertion order: last seen last)
+        if key[0] == "prompt":
+            prompts = [k for k in self._graphs if k[0] == "prompt"]
+            for k in prompts[:max(0, len(prompts) - self.max_prompt_graphs)]:
+                del self._graphs[k]

@@ -43,6 +43,9 @@ class DecoderModel:
         # whether a decode step may be recorded as a graph: every part must say so
         self.graph_safe = all(getattr(part, "graph_safe", True)
                               for part in [self.embedding, self.head] + self.blocks)
+        # ... and a short prompt step of a shape seen before
+        self.prompt_graph_safe = self.graph_safe and all(getattr(part, "prompt_graph_safe", False)
+                                                         for part in [self.embedding, self.head] + self.blocks)
 
     @property
     def embed(self) -> Optional[torch.Tensor]:

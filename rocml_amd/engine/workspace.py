@@ -22,6 +22,7 @@ class Workspace:
     def __init__(self, device, scratch_bytes: int = SCRATCH_BYTES):
         self.device = device
         self._buffers: Dict[str, torch.Tensor] = {}
+        self._views: Dict[tuple, torch.Tensor] = {}     # (name, type, shape) -> the view handed out last time
         self.generation = 0
         self._scratch_bytes = scratch_bytes
         self._scratch = None
@@ -32,6 +33,10 @@ class Workspace:
         self._prescaled = None
 
     def get(self, name: str, shape: Tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
+        # (a step asks for the same few views over and over; building one costs as much as a launch)
+        view = self._views.get((name, dtype, shape))
+        if view is not None:
+            return view
         n = math.prod(shape)
         key = f"{name}/{dtype}"
         buf = self._buffers.get(key)
@@ -39,7 +44,11 @@ class Workspace:
             buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
             self._buffers[key] = buf
             self.generation += 1
-        return buf[:n].view(shape)
+            self._views = {k: v for k, v in self._views.items() if (k[0], k[1]) != (name, dtype)}
+        view = buf[:n].view(shape)
+        if len(self._views) < 4096:
+            self._views[(name, dtype, shape)] = view
+        return view
 
     def scratch(self) -> torch.Tensor:
         """Device memory kernels may use for partial results of one launch.  Partial sums

@@ -40,6 +40,10 @@ class Attention(Mixer):
         self.q_dim = spec.n_heads * spec.head_dim
         self.kv_dim = spec.n_kv_heads * spec.head_dim
         self.position = build_position(spec.position, ctx) if spec.position is not None else None
+        # (what may be recorded as a graph: the attention's own launches always, its position
+        # encoding's if that part says so)
+        self.graph_safe = self.position is None or getattr(self.position, "graph_safe", True)
+        self.prompt_graph_safe = self.graph_safe and (self.position is None or getattr(self.position, "prompt_graph_safe", False))
         self.w_qkv: Optional[torch.Tensor] = None
         self.w_o: Optional[torch.Tensor] = None
         self.q_gain: Optional[torch.Tensor] = None

@@ -70,6 +70,11 @@ class Part:
     # False: forward() waits for the GPU or works on the host (reads a tensor back, loops over
     # tokens), so a decode step with this part cannot be recorded and replayed as a graph
     graph_safe = True
+    # True: the same holds for a step that brings several tokens per sequence: given the
+    # sequences' token counts and first positions, forward() launches the same device work every
+    # time and touches nothing on the host, so a short prompt step of a shape seen before may be
+    # replayed too.  A part has to say so itself.
+    prompt_graph_safe = False
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         return {}

@@ -27,6 +27,7 @@ class PreNormBlock(Part):
         self.ffn_norm = self.children["ffn_norm"]
         self.ffn = self.children["ffn"]
         self.graph_safe = all(getattr(c, "graph_safe", True) for c in self.children.values())
+        self.prompt_graph_safe = all(getattr(c, "prompt_graph_safe", False) for c in self.children.values())
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         return {f"{name}.{p}": spec for name, child in self.children.items()

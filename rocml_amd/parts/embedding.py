@@ -13,6 +13,8 @@ from .registry import register_embedding
 
 
 class TokenTable(Embedding):
+    prompt_graph_safe = True
+
     def __init__(self, spec: TokenTableSpec, ctx: BuildContext):
         self.vocab = spec.vocab
         self.hidden = spec.hidden

@@ -26,6 +26,7 @@ class NormLinearHead(Head):
         self.norm = build_norm(spec.norm, ctx)
         self.matrix: Optional[torch.Tensor] = None
         self.graph_safe = getattr(self.norm, "graph_safe", True)
+        self.prompt_graph_safe = getattr(self.norm, "prompt_graph_safe", False)
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         specs = {f"final_norm.{name}": p for name, p in self.norm.param_specs().items()}

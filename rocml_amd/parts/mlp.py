@@ -17,6 +17,7 @@ from .registry import register_feed_forward
 
 class GatedMlp(FeedForward):
     adds_only = True
+    prompt_graph_safe = True
 
     def __init__(self, spec: GatedMlpSpec, ctx: BuildContext):
         if spec.activation != "silu":

@@ -14,6 +14,8 @@ from .registry import register_norm
 
 
 class RMSNorm(Norm):
+    prompt_graph_safe = True
+
     def __init__(self, spec: NormSpec, ctx: BuildContext):
         self.size = spec.size
         self.eps = float(spec.eps)

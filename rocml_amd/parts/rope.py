@@ -14,6 +14,8 @@ from .registry import register_position
 
 
 class RopeNeox(PositionEncoding):
+    prompt_graph_safe = True
+
     def __init__(self, spec: RopeSpec, ctx: BuildContext):
         if spec.rot_dim % 2 != 0 or not 0 < spec.rot_dim <= spec.head_dim:
             raise ConfigError(f"rotary width {spec.rot_dim} must be even and at most the head size {spec.head_dim}")

@@ -234,3 +234,46 @@ def test_many_sequences_in_a_step(models, name, dtype, n_seqs):
     for s in slots:
         engine.release(s)
     engine.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_short_prompt_steps_of_a_shape_seen_before_are_replayed(models, dtype):
+    """A prompt step of a shape that came before (the same token counts and first positions) is
+    recorded the second time and replayed from then on; only the tables differ between replays:
+    other tokens, other wanted places, other slots and pages.  Every run must give what the plain
+    implementation gives, and other shapes in between must not disturb the recorded one."""
+    from rocml_amd.engine import StepEntry
+    path, cfg, weights = models["H"]
+    engine = _engine(path, dtype)
+    oracle_w = _oracle_weights(weights, dtype)
+    tol = TOL[dtype]
+
+    def once(seed, lengths, firsts, want_of):
+        """Sequences whose first ``firsts[i]`` tokens are already cached bring ``lengths[i]`` more."""
+        seqs = [helpers.random_tokens(f + n, cfg["vocab_size"], seed + i) for i, (n, f) in enumerate(zip(lengths, firsts))]
+        slots = [engine.new_sequence() for _ in seqs]
+        held = [(s, q[:f]) for s, q, f in zip(slots, seqs, firsts) if f]
+        if held:
+            engine.step([StepEntry(s, q, []) for s, q in held])
+        wants = [want_of(n) for n in lengths]
+        got = engine.step([StepEntry(s, q[f:], w) for s, q, f, w in zip(slots, seqs, firsts, wants)]).cpu()
+        expect = torch.cat([plain.forward(cfg, oracle_w, q)[[f + j for j in w]] for q, f, w in zip(seqs, firsts, wants)])
+        assert helpers.rel_to_max(got, expect) < tol, (seed, lengths, firsts)
+        for s in slots:
+            engine.release(s)
+
+    shape = ([17, 5, 40], [0, 0, 0])
+    for k in range(4):
+        once(700 + 10 * k, *shape, want_of=lambda n, k=k: [k % n, n - 1])
+        once(800 + 10 * k, [9], [0], want_of=lambda n: [n - 1])            # another shape in between
+    recorded = [key for key, entry in engine._graphs.items() if key[0] == "prompt" and entry[1] is not None]
+    assert ("prompt", (17, 5, 40), (0, 0, 0), 6, 1) in recorded and ("prompt", (9,), (0,), 1, 1) in recorded
+    # a continuation deep in a sequence, over a page border, is a shape of its own
+    for k in range(3):
+        once(900 + 10 * k, [30, 3], [50, 64], want_of=lambda n: [0, n - 1])
+    assert any(key[:3] == ("prompt", (30, 3), (50, 64)) and entry[1] is not None for key, entry in engine._graphs.items())
+    engine.cache.check()
+    # of the prompt shapes only the last few are kept
+    engine.max_prompt_graphs = 2
+    once(990, [4], [0], want_of=lambda n: [0])
+    assert sum(1 for key in engine._graphs if key[0] == "prompt") == 2
