@@ -285,7 +285,7 @@ __global__ void qk_norm_rope_append_kernel(
     TO* __restrict__ q_out, TO* __restrict__ kcache, TO* __restrict__ vcache,
     const int* __restrict__ block_table, int bt_width, const int* __restrict__ token_seq,
     const int* __restrict__ token_pos, int page_size, int write_kv, int n_splits, long long split_stride,
-    int rows_per_token) {
+    int rows_per_token, int pairing) {
     extern __shared__ float stage[];   // [QK_WAVES][d]
     int wave = threadIdx.x / WAVE;
     int lane = threadIdx.x & (WAVE - 1);
@@ -360,8 +360,15 @@ __global__ void qk_norm_rope_append_kernel(
             for (int j = 0; j < QK_PER_LANE; ++j) {
                 int e = lane + j * WAVE;
                 if (e < rot) {
-                    if (e < half) v[j] = v[j] * c[e] - mine[e + half] * s[e];
-                    else v[j] = mine[e - half] * s[e - half] + v[j] * c[e - half];
+                    if (pairing == 1) {
+                        // neighbours (2i, 2i + 1) are a pair, angle i
+                        float cs = c[e >> 1], sn = s[e >> 1], other = mine[e ^ 1];
+                        v[j] = (e & 1) ? other * sn + v[j] * cs : v[j] * cs - other * sn;
+                    } else if (e < half) {
+                        v[j] = v[j] * c[e] - mine[e + half] * s[e];
+                    } else {
+                        v[j] = mine[e - half] * s[e - half] + v[j] * c[e - half];
+                    }
                 }
             }
         }
@@ -504,7 +511,7 @@ v_append_tile_kernel(const TI* __restrict__ qkv, int ld, int n_tokens, int v_col
 
 ROCML_EXPORT int rocml_qk_norm_rope_append(
     const void* qkv, int in_dtype, int ld, int n_tokens, int hq, int hkv, int d, const float* q_gain,
-    const float* k_gain, float eps, const float* cos_t, const float* sin_t, int rot, void* q_out,
+    const float* k_gain, float eps, const float* cos_t, const float* sin_t, int rot, int pairing, void* q_out,
     void* kcache, void* vcache, int out_dtype, const int* block_table, int bt_width,
     const int* token_seq, const int* token_pos, int page_size, int write_kv, int n_splits,
     long long split_stride, hipStream_t stream) {
@@ -516,6 +523,7 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     ROCML_REQUIRE(ld >= (hq + 2 * hkv) * d || (!write_kv && ld >= hq * d),
                   "qk_norm_rope_append: row stride %d too small", ld);
     ROCML_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "qk_norm_rope_append: rot_dim %d must be even and <= %d", rot, d);
+    ROCML_REQUIRE(pairing == 0 || pairing == 1, "qk_norm_rope_append: pairing %d (0: halves, 1: neighbours)", pairing);
     ROCML_REQUIRE(!write_kv || (page_size > 0 && bt_width > 0 && block_table && kcache && vcache),
                   "qk_norm_rope_append: cache arguments missing");
     if (n_tokens == 0) return 0;
@@ -525,7 +533,8 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     long long rows = (long long)n_tokens * rows_per_token;
     int per_lane = d <= 64 ? 1 : d <= 128 ? 2 : d <= 256 ? 4 : 8;     // head values per lane
     // both values of a rotation pair in one lane: whole head rotated, d = per_lane * 64
-    bool local_pair = per_lane >= 2 && (rot == d || rot == 0) && d == per_lane * WAVE;
+    // (and the pairs are (e, e + d/2): neighbours as pairs go through LDS)
+    bool local_pair = per_lane >= 2 && (rot == 0 || (rot == d && pairing == 0)) && d == per_lane * WAVE;
     // many rows, none of them values: several rows per wave
     bool many_rows = local_pair && per_lane <= 4 && n_splits == 1 && n_tokens >= VT_TOKENS && (v_tiled || !write_kv);
     constexpr int MANY = 4;
@@ -535,7 +544,7 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     qk_norm_rope_append_kernel<TI, TO, N, LP><<<grid, EW_BLOCK, lds, stream>>>(                 \
         (const TI*)qkv, ld, n_tokens, hq, hkv, d, q_gain, k_gain, eps, cos_t, sin_t, rot,       \
         (TO*)q_out, (TO*)kcache, (TO*)vcache, block_table, bt_width, token_seq, token_pos,      \
-        page_size, write_kv, n_splits, split_stride, rows_per_token)
+        page_size, write_kv, n_splits, split_stride, rows_per_token, pairing)
 #define LAUNCH_ROWS(TI, TO, N)                                                                  \
     qk_norm_rope_rows_kernel<TI, TO, N, MANY><<<grid, EW_BLOCK, 0, stream>>>(                   \
         (const TI*)qkv, ld, n_tokens, hq, hkv, d, q_gain, k_gain, eps, rot ? cos_t : nullptr,   \

@@ -42,7 +42,6 @@ class StepContext:
     memo: Dict = field(default_factory=dict)
     block_tables: Dict = field(default_factory=dict)   # cache group name -> [B, width] int32
     want_rows: Optional[torch.Tensor] = None           # token rows whose logits are wanted
-    row_scale: Optional[object] = None                 # set around a part's forward: its input lacks this scale
 
     @property
     def is_decode(self) -> bool:

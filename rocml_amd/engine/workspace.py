@@ -27,10 +27,6 @@ class Workspace:
         self._scratch_bytes = scratch_bytes
         self._scratch = None
         self._pending = None
-        # the norm that will read the residual stream next, if its consumer can apply the norm's
-        # scale itself (set by the block around a part's forward); and what add_product made of it
-        self.next_norm = None
-        self._prescaled = None
 
     def get(self, name: str, shape: Tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
         # (a step asks for the same few views over and over; building one costs as much as a launch)
@@ -58,37 +54,6 @@ class Workspace:
             self.generation += 1
         self.flush_pending()
         return self._scratch
-
-    # -- products into the residual stream ------------------------------------------------------
-    def add_product(self, a: torch.Tensor, w: torch.Tensor, target: torch.Tensor) -> None:
-        """``target += a @ w.T``: how a part adds its result to the 32-bit residual stream.  The
-        product may be cut along K and its partial sums left for the next norm (``take_pending``),
-        or, when ``next_norm`` is set and the product is small enough, completed by one kernel
-        that also prepares that norm's output up to the rows' scale (``take_prescaled``)."""
-        from .. import ops
-        hint = self.next_norm
-        self._prescaled = None
-        if hint is not None and target.dtype == torch.float32 and hint.width == target.shape[1] \
-                and ops.gemm_residual_prescale_pays(a, w):
-            self.flush_pending()
-            rows = target.shape[0]
-            xg = self.get("residual.prepared", tuple(target.shape), torch.bfloat16)
-            parts = (target.shape[1] + ops.PRESCALE_TILE - 1) // ops.PRESCALE_TILE
-            ssq = self.get("residual.ssq", (rows, parts), torch.float32)
-            ops.gemm_residual_prescale(a, w, target, hint.gain, xg, ssq)
-            self._prescaled = (target.data_ptr(), hint.gain.data_ptr(), xg, ops.RowScale(ssq, hint.eps, hint.width))
-            return
-        splits = ops.gemm(a, w, target, accumulate=True, workspace=self.scratch(), defer=True)
-        if splits:
-            self.set_pending(target, splits)
-
-    def take_prescaled(self, target: torch.Tensor, gain: torch.Tensor):
-        """``(operand, row scale)`` if the last ``add_product`` into ``target`` prepared the norm
-        with this ``gain``; None otherwise (``target`` is complete then, or has pending sums)."""
-        hit, self._prescaled = self._prescaled, None
-        if hit is None or hit[0] != target.data_ptr() or hit[1] != gain.data_ptr():
-            return None
-        return hit[2], hit[3]
 
     # -- deferred split-K sums --------------------------------------------------------------
     # A product that was split along K and whose result is to be added to a tensor may leave
@@ -126,8 +91,6 @@ class Workspace:
 
     def drop_pending(self) -> None:
         self._pending = None
-        self._prescaled = None
-        self.next_norm = None
 
     def bytes(self) -> int:
         total = sum(b.numel() * b.element_size() for b in self._buffers.values())

@@ -31,7 +31,7 @@ _SIGNATURES = {
         "rocml_rmsnorm": [_P, _P, _P, _I, _P, _I, _I, _F, _P, _I, _LL, _P],
         "rocml_swiglu": [_P, _I, _P, _I, _I, _I, _I, _P],
         "rocml_rope_table": [_P, _P, _P, _P, _I, _I, _P],
-        "rocml_qk_norm_rope_append": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P, _P, _I, _P, _P, _P,
+        "rocml_qk_norm_rope_append": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P, _P, _I, _I, _P, _P, _P,
                                       _I, _P, _I, _P, _P, _I, _I, _I, _LL, _P],
         "rocml_add_into": [_P, _P, _I, _LL, _P],
     },
@@ -212,16 +212,23 @@ def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, cos: torch.Tenso
         _ptr(positions), _ptr(inv_freq), _ptr(cos), _ptr(sin), n, half, _stream()))
 
 
+ROPE_PAIRINGS = {"halves": 0, "neighbours": 1}
+
+
 def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,
                         q_gain: Optional[torch.Tensor], k_gain: Optional[torch.Tensor], eps: float,
                         cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rot_dim: int,
                         q_out: torch.Tensor, k_cache: Optional[torch.Tensor],
                         v_cache: Optional[torch.Tensor], block_table: Optional[torch.Tensor],
                         token_seq: torch.Tensor, token_pos: torch.Tensor, write_kv: bool = True,
-                        n_splits: int = 1) -> None:
+                        n_splits: int = 1, pairing: str = "halves") -> None:
     """``qkv`` is ``[T, ld]`` with q, k, v side by side (k and v may be absent when
     ``write_kv`` is false).  Keys are ``[pages, Hkv, page_size, D]``, values
-    ``[pages, Hkv, D, page_size]``."""
+    ``[pages, Hkv, D, page_size]``.  ``pairing``: which two values of the rotated width turn
+    together by the angle in column ``i`` of the tables: ``"halves"``, ``(i, i + rot_dim / 2)``,
+    or ``"neighbours"``, ``(2 i, 2 i + 1)``."""
+    if pairing not in ROPE_PAIRINGS:
+        raise KernelError(f"unknown rotation pairing {pairing!r}; known: {sorted(ROPE_PAIRINGS)}")
     _dev(qkv, q_gain, k_gain, cos, sin, q_out, k_cache, v_cache, block_table, token_seq, token_pos)
     split_stride = 0
     if n_splits > 1:                      # [splits, T, ld] split-K partial sums, added in the kernel
@@ -254,7 +261,7 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
         page_size, bt_width = k_cache.shape[2], block_table.shape[1]
     _check("elementwise", library("elementwise").rocml_qk_norm_rope_append(
         _ptr(qkv), _code(qkv), ld, n_tokens, n_heads, n_kv_heads, head_dim, _ptr(q_gain), _ptr(k_gain),
-        eps, _ptr(cos), _ptr(sin), rot_dim if cos is not None else 0, _ptr(q_out), _ptr(k_cache),
+        eps, _ptr(cos), _ptr(sin), rot_dim if cos is not None else 0, ROPE_PAIRINGS[pairing], _ptr(q_out), _ptr(k_cache),
         _ptr(v_cache), _code(q_out), _ptr(block_table), bt_width, _ptr(token_seq), _ptr(token_pos),
         page_size, 1 if write_kv else 0, n_splits, split_stride, _stream()))
 
@@ -444,12 +451,12 @@ def decode_splits(pairs: int, n_cus: int, most: int) -> int:
 
 
 def attention_decode_fusable(dtype: torch.dtype, n_heads: int, n_kv_heads: int, head_dim: int, page: int,
-                             rot_dim: Optional[int]) -> bool:
+                             rot_dim: Optional[int], pairing: str = "halves") -> bool:
     """Whether ``attention_decode_fused`` takes this layer: bfloat16 cache in pages of 64, a head
     size it has a kernel for, at most 16 query heads per kv head, and a rotation (if any) of the
-    whole head."""
+    whole head in pairs ``(i, i + head_dim / 2)``."""
     return (dtype == torch.bfloat16 and page == 64 and head_dim in FUSED_DECODE_HEAD_DIMS
-            and n_heads // n_kv_heads <= 16 and rot_dim in (None, head_dim))
+            and n_heads // n_kv_heads <= 16 and (rot_dim is None or (rot_dim == head_dim and pairing == "halves")))
 
 
 def attention_decode_fused(qkv: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,

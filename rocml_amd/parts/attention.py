@@ -19,6 +19,7 @@ from ..config.spec import AttentionSpec
 from ..errors import ConfigError
 from .base import BuildContext, KVCacheRequest, Mixer, ParamSpec
 from .registry import build_position, register_mixer
+from .residual import stream
 
 
 class Attention(Mixer):
@@ -40,6 +41,9 @@ class Attention(Mixer):
         self.q_dim = spec.n_heads * spec.head_dim
         self.kv_dim = spec.n_kv_heads * spec.head_dim
         self.position = build_position(spec.position, ctx) if spec.position is not None else None
+        self.pairing = getattr(self.position, "pairing", "halves")
+        if self.pairing not in ops.ROPE_PAIRINGS:
+            raise ConfigError(f"unknown rotation pairing {self.pairing!r}; known: {sorted(ops.ROPE_PAIRINGS)}")
         # (what may be recorded as a graph: the attention's own launches always, its position
         # encoding's if that part says so)
         self.graph_safe = self.position is None or getattr(self.position, "graph_safe", True)
@@ -89,7 +93,7 @@ class Attention(Mixer):
     def _fused_decode(self, step) -> bool:
         rot = None if self.position is None else self.position.rot_dim
         return step.max_new == 1 and ops.attention_decode_fusable(
-            self.dtype, self.spec.n_heads, self.spec.n_kv_heads, self.spec.head_dim, ops.FUSED_DECODE_PAGE, rot)
+            self.dtype, self.spec.n_heads, self.spec.n_kv_heads, self.spec.head_dim, ops.FUSED_DECODE_PAGE, rot, self.pairing)
 
     def takes_row_scale(self, step) -> bool:
         # only the decode kernel that reads the projection's sums itself applies a scale to them
@@ -132,19 +136,19 @@ class Attention(Mixer):
                                        s.n_heads, s.n_kv_heads, s.head_dim, s.scale, self.q_gain, self.k_gain, eps,
                                        cos, sin, write_kv=owns_cache, window=s.window, workspace=scratch[used:],
                                        max_len=step.max_len, n_splits=self._decode_splits(step, cache),
-                                       row_scale=step.row_scale)
+                                       row_scale=stream(step).row_scale)
         else:
-            if step.row_scale is not None:
+            if stream(step).row_scale is not None:
                 raise ConfigError("the attention was handed an input without its norm's scale in a step it cannot scale")
             q = ws.get("attn.q", (n, self.q_dim), self.dtype)
             ops.qk_norm_rope_append(qkv, s.n_heads, s.n_kv_heads, s.head_dim, self.q_gain, self.k_gain, eps,
                                     cos, sin, rot, q, cache.k, cache.v, cache.block_table, step.token_seq,
-                                    step.token_pos, write_kv=owns_cache, n_splits=max(splits, 1))
+                                    step.token_pos, write_kv=owns_cache, n_splits=max(splits, 1), pairing=self.pairing)
             ops.attention(q, o, cache.k, cache.v, cache.block_table, step.token_seq, step.token_pos,
                           s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, workspace=ws.scratch(),
                           cu_seqlens=step.cu_seqlens, max_new=step.max_new, q_counts=step.new_counts,
                           max_len=step.max_len, n_splits=self._decode_splits(step, cache))
-        ws.add_product(o, self.w_o, x_accum)
+        stream(step).add_product(o, self.w_o, x_accum)
 
 
 register_mixer("attention", Attention)

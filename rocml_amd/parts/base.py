@@ -130,8 +130,10 @@ class Norm(Part):
 class PositionEncoding(Part):
     """What the attention part asks of it: an attribute ``rot_dim`` (the leading width of a head
     that is rotated, even) and ``tables(step)`` returning ``(cos, sin)``, two 32-bit tensors
-    ``[tokens, rot_dim / 2]`` for the step's ``token_pos``; pair ``(i, i + rot_dim / 2)`` of a
-    head is rotated by the angle whose cosine and sine stand in column ``i``."""
+    ``[tokens, rot_dim / 2]`` for the step's ``token_pos``; the pair of a head that is rotated by
+    the angle whose cosine and sine stand in column ``i`` is ``(i, i + rot_dim / 2)`` with
+    ``pairing = "halves"`` and ``(2 i, 2 i + 1)`` with ``pairing = "neighbours"``."""
+    pairing = "halves"
 
     def tables(self, step: Any) -> Any:
         """Per-step tables for the step's token positions; computed once a step (``step.memo``
@@ -144,7 +146,8 @@ class Mixer(Part):
 
     def takes_row_scale(self, step: Any) -> bool:
         """Whether, in this step, forward() can take its input as ``bfloat16(x * gain)`` with the
-        norm's row scale still to be applied (``step.row_scale``, an ``ops.RowScale``) instead of
+        norm's row scale still to be applied (``parts.residual.stream(step).row_scale``, an
+        ``ops.RowScale``) instead of
         the normed input."""
         return False
 

@@ -12,6 +12,7 @@ import torch
 from ..config.spec import BlockSpec
 from .base import BuildContext, ParamSpec, Part
 from .registry import build_feed_forward, build_mixer, build_norm, register_block
+from .residual import stream
 
 
 class PreNormBlock(Part):
@@ -60,19 +61,20 @@ class PreNormBlock(Part):
         """``next_norm``: the hint of the norm that reads ``x`` after this block (``entry_hint`` of
         the block that runs next), or None."""
         ws = step.workspace
-        xn, step.row_scale = self._norm(step, self.mixer_norm, x)
+        rs = stream(step)
+        xn, rs.row_scale = self._norm(step, self.mixer_norm, x)
         if not getattr(self.mixer, "adds_only", False):
             ws.flush_pending()
-        ws.next_norm = self._hint(step, self.ffn_norm, self.ffn)
+        rs.next_norm = self._hint(step, self.ffn_norm, self.ffn)
         self.mixer.forward(step, xn, x, cache, owns_cache)
-        ws.next_norm = None
-        xn, step.row_scale = self._norm(step, self.ffn_norm, x)
+        rs.next_norm = None
+        xn, rs.row_scale = self._norm(step, self.ffn_norm, x)
         if not getattr(self.ffn, "adds_only", False):
             ws.flush_pending()
-        ws.next_norm = next_norm
+        rs.next_norm = next_norm
         self.ffn.forward(step, xn, x)
-        ws.next_norm = None
-        step.row_scale = None
+        rs.next_norm = None
+        rs.row_scale = None
 
     @staticmethod
     def _hint(step, norm, consumer):
@@ -89,7 +91,7 @@ class PreNormBlock(Part):
         completed."""
         ws = step.workspace
         gain = getattr(norm, "gain", None)
-        prepared = ws.take_prescaled(x, gain) if gain is not None else None
+        prepared = stream(step).take_prescaled(x, gain) if gain is not None else None
         if prepared is not None:
             return prepared
         xn = ws.get("block.xn", tuple(x.shape), self.dtype)

@@ -13,6 +13,7 @@ from ..config.spec import GatedMlpSpec
 from ..errors import ConfigError
 from .base import BuildContext, FeedForward, ParamSpec
 from .registry import register_feed_forward
+from .residual import stream
 
 
 class GatedMlp(FeedForward):
@@ -57,14 +58,14 @@ class GatedMlp(FeedForward):
         ws = step.workspace
         h = ws.get("mlp.h", (n, s.intermediate), self.dtype)
         if self.fused:
-            ops.gemm(xn, self.w_gate_up, h, workspace=ws.scratch(), epilogue="swiglu", row_scale=step.row_scale)
+            ops.gemm(xn, self.w_gate_up, h, workspace=ws.scratch(), epilogue="swiglu", row_scale=stream(step).row_scale)
         else:
-            if step.row_scale is not None:
+            if stream(step).row_scale is not None:
                 raise ConfigError("the feed-forward was handed an input without its norm's scale in a step it cannot scale")
             gate_up = ws.get("mlp.gate_up", (n, 2 * s.intermediate), torch.float32)
             ops.gemm(xn, self.w_gate_up, gate_up, workspace=ws.scratch())
             ops.swiglu(gate_up, h, interleaved=True)
-        ws.add_product(h, self.w_down, x_accum)
+        stream(step).add_product(h, self.w_down, x_accum)
 
 
 register_feed_forward("gated_mlp", GatedMlp)

@@ -95,7 +95,17 @@ def test_add_into():
     assert torch.equal(x, want)
 
 
-def _qkv_case(tokens, hq, hkv, d, pos_base, theta, rot, norm, dtype, seed=0, splits=1):
+def _rope_neighbours(x, positions, theta):
+    """The rotation with neighbours as pairs: values (2i, 2i + 1) of a head turn by the angle
+    pos * theta^(-2i/D).  It is the rotation over halves applied to the head with its even
+    values first and its odd values behind them."""
+    d = x.shape[-1]
+    order = list(range(0, d, 2)) + list(range(1, d, 2))
+    back = [order.index(i) for i in range(d)]
+    return plain.rope_neox(x[..., order], positions, theta)[..., back]
+
+
+def _qkv_case(tokens, hq, hkv, d, pos_base, theta, rot, norm, dtype, seed=0, splits=1, pairing="halves"):
     """Runs the fused kernel on one sequence whose pages are handed out backwards; returns
     (q, k rows, v rows) read back from q_out and the cache, and the plain expectation."""
     g = torch.Generator().manual_seed(seed)
@@ -127,15 +137,16 @@ def _qkv_case(tokens, hq, hkv, d, pos_base, theta, rot, norm, dtype, seed=0, spl
     ops.qk_norm_rope_append(fed, hq, hkv, d, qg.cuda() if norm else None, kg.cuda() if norm else None, eps,
                             cos, sin, rot, q_out, kc, vc, table.cuda(),
                             torch.zeros(tokens, dtype=torch.int32).cuda(),
-                            torch.tensor(positions, dtype=torch.int32).cuda(), n_splits=splits)
+                            torch.tensor(positions, dtype=torch.int32).cuda(), n_splits=splits, pairing=pairing)
     q = qkv[:, :hq * d].reshape(tokens, hq, d).double()
     k = qkv[:, hq * d:(hq + hkv) * d].reshape(tokens, hkv, d).double()
     v = qkv[:, (hq + hkv) * d:].reshape(tokens, hkv, d).double()
     if norm:
         q, k = plain.rmsnorm(q, qg.double(), eps), plain.rmsnorm(k, kg.double(), eps)
     if rot:
-        q = torch.cat([plain.rope_neox(q[..., :rot], positions, theta), q[..., rot:]], -1)
-        k = torch.cat([plain.rope_neox(k[..., :rot], positions, theta), k[..., rot:]], -1)
+        turn = plain.rope_neox if pairing == "halves" else _rope_neighbours
+        q = torch.cat([turn(q[..., :rot], positions, theta), q[..., rot:]], -1)
+        k = torch.cat([turn(k[..., :rot], positions, theta), k[..., rot:]], -1)
     got_k = torch.stack([kc[table[0, p // page], :, p % page].cpu() for p in positions]).double()
     got_v = torch.stack([vc[table[0, p // page], :, :, p % page].cpu() for p in positions]).double()
     return q_out.cpu().double().reshape(tokens, hq, d), got_k, got_v, q, k, v, (kc, vc, table, positions)
@@ -161,6 +172,22 @@ def test_qk_norm_rope_append(tokens, hq, hkv, d, pos_base, rot, norm):
     assert float((gq - q).abs().max()) < 8e-3 * float(q.abs().max())
     assert float((gk - k).abs().max()) < 8e-3 * float(k.abs().max())
     assert float((gv - _bf16(v)).abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("tokens,hq,hkv,d,pos_base,rot,norm", [
+    (10, 3, 3, 16, 5, 16, True), (70, 4, 2, 48, 100, 48, True), (5, 2, 2, 128, 60, 64, True),
+    (3, 8, 2, 128, 60, 128, True), (150, 4, 2, 128, 37, 128, False), (2, 1, 1, 264, 1, 264, True)])
+def test_qk_norm_rope_append_with_neighbours_as_pairs(tokens, hq, hkv, d, pos_base, rot, norm):
+    """The other pairing of the rotation: (2i, 2i + 1) instead of (i, i + rot/2); a wrong partner,
+    a wrong angle column or a wrong sign fails it."""
+    for dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 8e-3)):
+        gq, gk, gv, q, k, v, _ = _qkv_case(tokens, hq, hkv, d, pos_base, 1e4, rot, norm, dtype, pairing="neighbours")
+        assert float((gq - q).abs().max()) < tol * max(1.0, float(q.abs().max()))
+        assert float((gk - k).abs().max()) < tol * max(1.0, float(k.abs().max()))
+    *_, q_halves, k_halves, _, _ = _qkv_case(tokens, hq, hkv, d, pos_base, 1e4, rot, norm, torch.float32)
+    assert float((q - q_halves).abs().max()) > 1e-2            # (the two pairings do differ on this input)
+    with pytest.raises(Exception, match="pairing"):
+        _qkv_case(2, 1, 1, 16, 0, 1e4, 16, True, torch.float32, pairing="thirds")
 
 
 @pytest.mark.parametrize("splits", [2, 5, 8])

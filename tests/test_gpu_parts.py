@@ -311,8 +311,13 @@ def _toy_routed_and_position():
                 step.memo[("toy_slowed_rope", self.spec)] = hit
             return hit
 
+    class NeighbourRope(SlowedRope):
+        """The same angles, but the values (2i, 2i + 1) of a head turn together."""
+        pairing = "neighbours"
+
     register_feed_forward("toy_routed", RoutedFfn)
     register_position("toy_slowed_rope", SlowedRope)
+    register_position("toy_neighbour_rope", NeighbourRope)
 
 
 def test_toy_routed_feed_forward_and_toy_position_encoding():
@@ -373,6 +378,58 @@ def test_toy_routed_feed_forward_and_toy_position_encoding():
     assert helpers.rel_to_max(helpers.run_tail_by_one(engine, b, 12), rb) < 1e-4
     got = helpers.run_batch(engine, [a, b], [35, 4])
     assert helpers.rel_to_max(got[0], ra) < 1e-4 and helpers.rel_to_max(got[1], rb) < 1e-4
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 1e-4), ("bfloat16", 2e-2)])
+def test_toy_position_encoding_that_pairs_neighbours(dtype, tol):
+    """A position encoding whose pairs are (2i, 2i + 1): the part only says so (``pairing``); the
+    attention's kernels take the pairing as a parameter, and the decode kernel that rotates inside
+    the attention, which knows halves only, is not taken (head size 64 in bfloat16 would take it)."""
+    _toy_routed_and_position()
+    hidden, d = 48, 64
+    rope = SlowedRopeSpec(d, d, 1e4, 1.0, kind="toy_neighbour_rope")
+    att = AttentionSpec(hidden=hidden, n_heads=4, n_kv_heads=2, head_dim=d, scale=1 / math.sqrt(d), window=None,
+                        qk_norm=NormSpec(d, 1e-5), position=rope)
+    spec = _spec([_block(hidden, att), _block(hidden, att)], [ScheduleEntry(0), ScheduleEntry(1)], hidden, 97)
+    engine, w = _engine(spec, dtype, seed=12)
+    assert not engine.model.blocks[0].mixer._fused_decode(type("S", (), {"max_new": 1})())
+    if dtype == "bfloat16":
+        w = {k: (v if v.dim() == 1 else v.to(torch.bfloat16).double()) for k, v in w.items()}
+
+    def turn(x, positions):
+        order = list(range(0, d, 2)) + list(range(1, d, 2))
+        back = [order.index(i) for i in range(d)]
+        return plain.rope_neox(x[..., order], positions, rope.theta)[..., back]
+
+    def reference(tokens):
+        x = w["embed.weight"][tokens]
+        pos = list(range(len(tokens)))
+        t = len(tokens)
+        for i in range(2):
+            pre = f"layers.{i}."
+            xn = plain.rmsnorm(x, w[pre + "mixer_norm.weight"], 1e-5)
+            q = plain.rmsnorm((xn @ w[pre + "mixer.q_proj.weight"].t()).reshape(t, 4, d), w[pre + "mixer.q_norm.weight"], 1e-5)
+            k = plain.rmsnorm((xn @ w[pre + "mixer.k_proj.weight"].t()).reshape(t, 2, d), w[pre + "mixer.k_norm.weight"], 1e-5)
+            v = (xn @ w[pre + "mixer.v_proj.weight"].t()).reshape(t, 2, d)
+            o = plain.causal_attention(turn(q, pos), turn(k, pos), v, att.scale, None)
+            x = x + o.reshape(t, -1) @ w[pre + "mixer.o_proj.weight"].t()
+            xn = plain.rmsnorm(x, w[pre + "ffn_norm.weight"], 1e-5)
+            x = x + plain.swiglu(xn @ w[pre + "ffn.gate_proj.weight"].t(), xn @ w[pre + "ffn.up_proj.weight"].t()) \
+                @ w[pre + "ffn.down_proj.weight"].t()
+        return plain.rmsnorm(x, w["final_norm.weight"], 1e-5) @ w["embed.weight"].t()
+
+    a, b = helpers.random_tokens(70, 97, 19), helpers.random_tokens(9, 97, 20)
+    ra, rb = reference(a), reference(b)
+    assert helpers.rel_to_max(helpers.run_whole(engine, a), ra) < tol
+    assert helpers.rel_to_max(helpers.run_tail_by_one(engine, b, 6), rb) < tol
+    got = helpers.run_batch(engine, [a, b], [60, 3])
+    assert helpers.rel_to_max(got[0], ra) < tol and helpers.rel_to_max(got[1], rb) < tol
+    # (and the pairing does matter: with halves as pairs the logits are others)
+    wrong = SlowedRopeSpec(d, d, 1e4, 1.0)
+    att2 = AttentionSpec(hidden=hidden, n_heads=4, n_kv_heads=2, head_dim=d, scale=1 / math.sqrt(d), window=None,
+                         qk_norm=NormSpec(d, 1e-5), position=wrong)
+    other, _ = _engine(_spec([_block(hidden, att2), _block(hidden, att2)], [ScheduleEntry(0), ScheduleEntry(1)], hidden, 97), dtype, seed=12)
+    assert helpers.rel_to_max(helpers.run_whole(other, a), ra) > 10 * tol
 
 
 # ---- a toy embedding with learned positions and a toy head with a soft cap ------------------
