@@ -277,3 +277,71 @@ def test_short_prompt_steps_of_a_shape_seen_before_are_replayed(models, dtype):
     engine.max_prompt_graphs = 2
     once(990, [4], [0], want_of=lambda n: [0])
     assert sum(1 for key in engine._graphs if key[0] == "prompt") == 2
+
+
+LONG = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "vocab_size": 300,
+        "hidden_size": 64, "intermediate_size": 96, "num_hidden_layers": 1,
+        "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 64,
+        "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True,
+        "max_position_embeddings": 40960, "hidden_act": "silu", "attention_bias": False}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_prompt_of_33000_tokens_and_decoding_behind_it(tmp_path, dtype):
+    """A sequence as long as the long-context figures are quoted for: a prompt of 33,000 tokens
+    (five pieces of the engine's cut, a block table of 516 pages and more, the most key splits in
+    the decode steps), then tokens one by one across a page border, a short sequence beside it.
+    The model has one layer, so keys and values of every position follow from the embeddings
+    alone and the plain implementation's parts give the logits of the last places without the
+    33,000 x 33,000 scores of a whole pass."""
+    import math
+    from rocml_amd.engine import Engine, StepEntry
+    from rocml_amd.weights import load_model
+    path = helpers.make_model_dir(tmp_path, LONG, 31, torch.float32)
+    cfg, weights = helpers.read_config(path), helpers.read_weights(path)
+    w = {k: v.double() for k, v in _oracle_weights(weights, dtype).items()}
+    n_prompt, n_decode, last = 33000, 40, 6
+    toks = helpers.random_tokens(n_prompt + n_decode, cfg["vocab_size"], 41)
+    short = helpers.random_tokens(20 + n_decode, cfg["vocab_size"], 42)
+
+    def last_logits(tokens, places):
+        d, hq, hkv, eps = cfg["head_dim"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["rms_norm_eps"]
+        t = len(tokens)
+        p = "model.layers.0."
+        x = plain.embedding(w["model.embed_tokens.weight"], tokens)
+        xn = plain.rmsnorm(x, w[p + "input_layernorm.weight"], eps)
+        pos = list(range(t))
+        k = plain.rope_neox(plain.rmsnorm(plain.linear(xn, w[p + "self_attn.k_proj.weight"]).reshape(t, hkv, d),
+                                          w[p + "self_attn.k_norm.weight"], eps), pos, cfg["rope_theta"])
+        v = plain.linear(xn, w[p + "self_attn.v_proj.weight"]).reshape(t, hkv, d)
+        rows = torch.tensor(places)
+        q = plain.rope_neox(plain.rmsnorm(plain.linear(xn[rows], w[p + "self_attn.q_proj.weight"]).reshape(len(places), hq, d),
+                                          w[p + "self_attn.q_norm.weight"], eps), places, cfg["rope_theta"])
+        o = torch.zeros(len(places), hq, d, dtype=torch.float64)
+        for i, place in enumerate(places):             # the attention's formula, row by row (plain.causal_attention)
+            for h in range(hq):
+                s = (k[:place + 1, h // (hq // hkv)] @ q[i, h]) / math.sqrt(d)
+                e = torch.exp(s - s.max())
+                o[i, h] = (e @ v[:place + 1, h // (hq // hkv)]) / e.sum()
+        x = x[rows] + plain.linear(o.reshape(len(places), hq * d), w[p + "self_attn.o_proj.weight"])
+        x = x + plain.mlp_block(plain.rmsnorm(x, w[p + "post_attention_layernorm.weight"], eps), w, p)
+        return plain.linear(plain.rmsnorm(x, w["model.norm.weight"], eps), w["model.embed_tokens.weight"])
+
+    engine = Engine(load_model(path, dtype=dtype, device="cuda:0"), max_tokens=(n_prompt + n_decode + 64) // 64 * 64 + 128,
+                    max_seqs=2)
+    a, b = engine.new_sequence(), engine.new_sequence()
+    places = list(range(n_prompt - last, n_prompt))
+    got = [engine.step([StepEntry(a, toks[:n_prompt], places), StepEntry(b, short[:20], [19])]).cpu()]
+    for i in range(n_decode):
+        got.append(engine.step([StepEntry(a, [toks[n_prompt + i]], [0]), StepEntry(b, [short[20 + i]], [0])]).cpu())
+    assert engine.cache.table_width([a, b]) >= 516
+    long_rows = torch.cat([got[0][:last]] + [g[:1] for g in got[1:]])
+    short_rows = torch.cat([got[0][last:]] + [g[1:] for g in got[1:]])
+    want = last_logits(toks, places + list(range(n_prompt, n_prompt + n_decode)))
+    tol = TOL[dtype]
+    assert helpers.rel_to_max(long_rows, want) < tol and helpers.per_position(long_rows, want) < 5 * tol
+    want_short = last_logits(short, list(range(19, 20 + n_decode)))
+    assert helpers.rel_to_max(short_rows, want_short) < tol
+    engine.release(a)
+    engine.release(b)
+    engine.cache.check()
