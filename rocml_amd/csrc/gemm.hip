@@ -9,7 +9,8 @@
 ROCML_LAST_ERROR_FN(gemm)
 
 enum GemmAlgo : int { ALGO_AUTO = 0, ALGO_PLAIN = 1, ALGO_MFMA_TILE = 2, ALGO_MFMA_SKINNY = 3, ALGO_MFMA_KPAR = 4,
-                      ALGO_MFMA_TILE256 = 5, ALGO_MFMA_TILE192 = 6 };
+                      ALGO_MFMA_TILE256 = 5, ALGO_MFMA_TILE192 = 6, ALGO_MFMA_TILE128X192 = 7, ALGO_MFMA_TILE256X96 = 8,
+                      ALGO_MFMA_TILE64X256 = 9 };
 
 static int round_up(int a, int b) { return (a + b - 1) / b * b; }
 
@@ -21,7 +22,7 @@ static int allow_lds(K kernel, int bytes, const char* name) {
     return 0;
 }
 
-struct SplitPlan { int defer; int* deferred; RowScale rs; };
+struct SplitPlan { int defer; int* deferred; RowScale rs; int max_splits; };   // max_splits: the most K pieces the caller wants
 
 template <int EPI, typename T>
 static int launch_mfma_tile_as(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m,
@@ -55,17 +56,67 @@ static int launch_mfma_tile_as(const void* x, int ldx, const void* w, int ldw, v
     return 0;
 }
 
-// shape: 0 = choose, 1 = 128x128 tiles, 2 = 256x256, 3 = 256x192.  The choice is made on an
-// estimate of the time.  A CU holds one big tile or two small ones; per 64-wide K stage a CU
-// that is kept busy needs about 2.0 us for a 256x256 tile, 1.62 us for a 256x192 one and 0.78 us
-// for a small one (measured in the model, weights from HBM: about 1060, 980 and 700 TFLOP/s; the
-// wider a wave's own tile and the more waves share an operand, the fewer LDS bytes per product).
-// What counts is the CU with the most tiles: 6144 columns are 24 tiles of 256, which with 2048
-// rows leave a quarter of the chip idle, or 32 tiles of 192, which fill it.  A
-// product with few tiles (few rows, or a narrow output) leaves most CUs idle while a few walk
-// through all of K: then K is cut into up to 8 pieces, each the work of a block of its own,
-// at the price of writing and reading the 32-bit partial sums once more.  No estimate may go
-// below the time the weights need to arrive.
+// The tile shapes of the many-rows kernel, as rows x columns of a block's tile: 128x128 (four waves
+// of 64x64, two blocks a CU), 256x256 (eight waves of 128x64), 256x192 (eight of 64x96), 128x192
+// (four of 64x96), 256x96 (four of 64x96, the whole of up to 256 rows against a narrow strip of
+// weights) and 64x256 (four of 64x64 side by side, for products of few rows).
+using GemmTile128x192 = GemmTile<2, 2, 2, 3>;
+using GemmTile256x96 = GemmTile<4, 1, 2, 3>;
+using GemmTile64x256 = GemmTile<1, 4, 2, 2>;
+
+// What a tile shape costs: microseconds per 64-wide K stage for a CU that holds as many blocks of it
+// as fit (`cap`), when half the chip or less is at work (`light`) and when all of it is (`full`: the
+// memory system is shared and the clock drops under load), and, for the shape of which two fit,
+// for a CU that holds one alone.  Measured on the Qwen3-8B and 14B products at 80 to 8192 rows.
+struct TileKind { int bm, bn, cap; double light, full, alone; int shape; };
+static const TileKind TILE_KINDS[] = {
+    {128, 128, 2, 1.21, 1.25, 0.88, 1}, {256, 256, 1, 1.55, 1.85, 0.0, 2}, {256, 192, 1, 1.22, 1.50, 0.0, 3},
+    {128, 192, 1, 1.00, 1.04, 0.0, 4},  {256, 96, 1, 1.03, 1.12, 0.0, 5},  {64, 256, 1, 0.93, 1.05, 0.0, 6}};
+
+// An estimate of a product's time in microseconds with tiles of `kind` and K cut into `pieces`
+// (each piece the work of a block of its own, 32-bit partial sums written once here and read once
+// by whoever adds them): the rounds of blocks the chip holds at a time, each round as long as its
+// K stages at the rate of the CUs' load, but no shorter than the busiest CU needs to pull its
+// blocks' operands (36 GB/s a CU: with few rows it is the weights' arrival that a block waits for,
+// and more, smaller blocks pull more at a time); a fixed part for the launch; the bytes the
+// epilogue moves; never less than the weights need to arrive at all.  The constants were fitted
+// to measurements of 103 products (the Qwen3-8B, 14B and 0.6B shapes at 52 to 8192 rows, six tile
+// shapes, one to eight pieces): the choice made on this estimate is 0.9 % behind the best choice
+// on average and within 5 % for nine in ten.
+static double tile_cost(const TileKind& kind, int pieces, int m, int n, int k, int epi, int cus) {
+    long long tiles = (long long)ceil_div(m, kind.bm) * ceil_div(n, kind.bn);
+    int k_per_piece = round_up(ceil_div(k, pieces), GM_BK);
+    pieces = ceil_div(k, k_per_piece);
+    long long blocks = tiles * pieces, slots = (long long)cus * kind.cap;
+    double stages = (double)(k_per_piece / GM_BK);
+    auto stage_us = [&](long long together) {          // blocks on the chip at the same time, at most `slots`
+        double share = (double)together / (double)cus;
+        if (kind.cap == 2 && together <= cus) return kind.alone * (1.0 + 0.2 * (share > 0.5 ? share - 0.5 : 0.0));
+        double busy = (double)together / (double)slots;
+        double w = busy <= 0.5 ? 0.0 : busy >= 1.0 ? 1.0 : (busy - 0.5) * 2.0;
+        return kind.light + (kind.full - kind.light) * w;
+    };
+    long long rounds = blocks / slots, rest = blocks % slots;
+    double t = (double)rounds * stages * stage_us(slots) + (rest ? stages * stage_us(rest) : 0.0);
+    double pulled = (double)(kind.bn + (m < kind.bm ? m : kind.bm)) * k_per_piece * 2.0 * (double)ceil_div(blocks, (long long)cus);
+    if (t < pulled / 36.0e3) t = pulled / 36.0e3;
+    t += 3.0;
+    double moved = epi == EPI_SWIGLU ? (double)m * n
+                   : pieces > 1      ? (double)m * n * 4.0 * pieces
+                                     : (double)m * n * 4.0 * (epi == EPI_ACC ? 2.0 : 1.0);
+    t += moved / 2.0e6;
+    double floor_us = (double)n * k * 2.0 / 5.5e6;                  // the weights at 5.5 TB/s
+    if (t < floor_us) t = floor_us;
+    if (pieces > 1) t += (double)pieces * m * n * 4.0 / 5.0e6;      // the partial sums read again
+    return t;
+}
+
+// shape: 0 = choose, else a TileKind's number (then K stays whole).  The choice is the smallest
+// estimate over shapes and pieces.  What counts is the CU with the most work: 6144 columns are 24
+// tiles of 256, which with 2048 rows leave a quarter of the chip idle, or 32 tiles of 192, which
+// fill it; a product of 256 rows and 24576 columns is 384 tiles of 128x128, one and a half to a
+// CU, or 256 of 128x192, one each.  A product with few tiles (few rows, or a narrow output)
+// leaves most CUs idle while a few walk through all of K: then K is cut into up to 8 pieces.
 template <int EPI>
 static int launch_mfma_tile(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m,
                             int n, int k, int shape, void* workspace, long long workspace_bytes, SplitPlan plan,
@@ -74,29 +125,24 @@ static int launch_mfma_tile(const void* x, int ldx, const void* w, int ldw, void
     const int cus = cu_count();
     if (shape == 0) {
         double best = 1e30;
-        // rows and columns of a tile, microseconds per 64-wide K stage, the shape's number
-        static const struct { int bm, bn; double stage_us; int shape; } kinds[] = {
-            {128, 128, 0.78, 1}, {256, 256, 2.0, 2}, {256, 192, 1.62, 3}};
-        for (const auto& kind : kinds) {
-            long long tiles = (long long)ceil_div(m, kind.bm) * ceil_div(n, kind.bn);
-            for (int pieces = 1; pieces <= 8; ++pieces) {
-                if (pieces > 1 && (EPI == EPI_SWIGLU || k / pieces < 512 || !workspace ||
+        for (const auto& kind : TILE_KINDS) {
+            for (int pieces = 1; pieces <= 8 && pieces <= plan.max_splits; ++pieces) {
+                if (pieces > 1 && (EPI == EPI_SWIGLU || k / pieces < 256 || !workspace ||
                                    (long long)pieces * m * n * (long long)sizeof(float) > workspace_bytes))
                     break;
-                long long blocks = tiles * pieces;
-                double per_cu = (double)ceil_div(blocks, cus);          // tiles of the busiest CU
-                double stages = (double)ceil_div(ceil_div(k, pieces), GM_BK);
-                double t = per_cu * stages * kind.stage_us + 4.0;
-                if (pieces > 1) t += (double)pieces * m * n * 8.0 / 4.0e6;   // partial sums out and in, 4 TB/s
-                double floor_us = (double)n * k * 2.0 / 5.5e6;               // the weights at 5.5 TB/s
-                if (t < floor_us) t = floor_us;
+                double t = tile_cost(kind, pieces, m, n, k, EPI, cus);
                 if (t < best) { best = t; shape = kind.shape; splits = pieces; }
             }
         }
     }
-    if (shape == 3) return launch_mfma_tile_as<EPI, GemmTile192>(x, ldx, w, ldw, out, ldo, m, n, k, splits, workspace, plan, stream);
-    if (shape == 2) return launch_mfma_tile_as<EPI, GemmTile256>(x, ldx, w, ldw, out, ldo, m, n, k, splits, workspace, plan, stream);
-    return launch_mfma_tile_as<EPI, GemmTile128>(x, ldx, w, ldw, out, ldo, m, n, k, splits, workspace, plan, stream);
+    switch (shape) {
+        case 6: return launch_mfma_tile_as<EPI, GemmTile64x256>(x, ldx, w, ldw, out, ldo, m, n, k, splits, workspace, plan, stream);
+        case 5: return launch_mfma_tile_as<EPI, GemmTile256x96>(x, ldx, w, ldw, out, ldo, m, n, k, splits, workspace, plan, stream);
+        case 4: return launch_mfma_tile_as<EPI, GemmTile128x192>(x, ldx, w, ldw, out, ldo, m, n, k, splits, workspace, plan, stream);
+        case 3: return launch_mfma_tile_as<EPI, GemmTile192>(x, ldx, w, ldw, out, ldo, m, n, k, splits, workspace, plan, stream);
+        case 2: return launch_mfma_tile_as<EPI, GemmTile256>(x, ldx, w, ldw, out, ldo, m, n, k, splits, workspace, plan, stream);
+        default: return launch_mfma_tile_as<EPI, GemmTile128>(x, ldx, w, ldw, out, ldo, m, n, k, splits, workspace, plan, stream);
+    }
 }
 
 // The two-steps-ahead kernel on a product that cannot be cut along K (the gated product), with
@@ -185,23 +231,24 @@ static double block_cost(BlockChoice c, int m, int row_tiles, int n, int cus) {
 }
 
 static BlockChoice choose_blocks(BlockChoice usual, int m, int row_tiles, int n, int k, int cus,
-                                 long long workspace_bytes, int skip_from, int skip_to) {
+                                 long long workspace_bytes, int skip_from, int skip_to, int max_splits) {
     // (a step asks for the same few products over and over: the last answers are kept)
     // (the answer depends on the usual blocks and on the skipped wave counts too, which differ
     // between the callers that share this table)
-    struct Kept { int m, row_tiles, n, k, cus; long long workspace_bytes; BlockChoice usual; int skip_from, skip_to;
+    struct Kept { int m, row_tiles, n, k, cus; long long workspace_bytes; BlockChoice usual; int skip_from, skip_to, max_splits;
                   BlockChoice choice; bool set; };
     static thread_local Kept kept[64];
     Kept& slot = kept[((unsigned)n * 31u + (unsigned)k * 7u + (unsigned)m) % 64u];
     if (slot.set && slot.m == m && slot.row_tiles == row_tiles && slot.n == n && slot.k == k && slot.cus == cus &&
         slot.workspace_bytes == workspace_bytes && slot.usual.waves == usual.waves && slot.usual.splits == usual.splits &&
-        slot.usual.k_per_split == usual.k_per_split && slot.skip_from == skip_from && slot.skip_to == skip_to)
+        slot.usual.k_per_split == usual.k_per_split && slot.skip_from == skip_from && slot.skip_to == skip_to &&
+        slot.max_splits == max_splits)
         return slot.choice;
     BlockChoice best = usual;
     double best_cost = 1e30;
     for (int kps = GS_KC; kps < k + GS_KC; kps += GS_KC) {
         int splits = ceil_div(k, kps);
-        if (splits > 16) continue;
+        if (splits > max_splits) continue;
         if (splits > 1 && (kps < 2 * GS_KC || (long long)splits * m * n * (long long)sizeof(float) > workspace_bytes)) continue;
         for (int waves = 2; waves <= 16; ++waves) {
             if (waves >= skip_from && waves <= skip_to) continue;
@@ -216,7 +263,7 @@ static BlockChoice choose_blocks(BlockChoice usual, int m, int row_tiles, int n,
     // the usual blocks (four or eight waves, about two blocks or one a CU) unless the estimate
     // promises a clear gain: it is rough, and they are what the kernels were tuned with
     BlockChoice choice = best_cost < 0.93 * block_cost(usual, m, row_tiles, n, cus) ? best : usual;
-    slot = Kept{m, row_tiles, n, k, cus, workspace_bytes, usual, skip_from, skip_to, choice, true};
+    slot = Kept{m, row_tiles, n, k, cus, workspace_bytes, usual, skip_from, skip_to, max_splits, choice, true};
     return choice;
 }
 
@@ -265,7 +312,7 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
     int splits = target / blocks_n;
     int by_k = k / 512;
     if (splits > by_k) splits = by_k;
-    if (splits > 16) splits = 16;
+    if (splits > plan.max_splits) splits = plan.max_splits;
     if (splits < 1 || narrow) splits = 1;
     long long per_split = (long long)m * n * sizeof(float);
     if (splits > 1 && (long long)splits * per_split > workspace_bytes)
@@ -276,7 +323,7 @@ static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* o
     dim3 grid(blocks_n, splits);
     if (!narrow && workspace) {
         BlockChoice usual{WIDE, splits, k_per_split};
-        BlockChoice c = choose_blocks(usual, m, MT, n, k, cus, workspace_bytes, MT == 4 ? 13 : 17, MT == 4 ? 15 : 17);
+        BlockChoice c = choose_blocks(usual, m, MT, n, k, cus, workspace_bytes, MT == 4 ? 13 : 17, MT == 4 ? 15 : 17, plan.max_splits);
         if (c.splits > 1 && (c.waves != usual.waves || c.splits != usual.splits)) {
             int rc = 1;
             switch (c.waves) {
@@ -338,7 +385,7 @@ static int launch_kpar(const void* x, int ldx, const void* w, int ldw, void* out
     int splits = 4 * cu_count() / n_tiles;
     int by_k = k / 1024;
     if (splits > by_k) splits = by_k;
-    if (splits > 16) splits = 16;
+    if (splits > plan.max_splits) splits = plan.max_splits;
     if (splits < 1 || EPI == EPI_SWIGLU) splits = 1;
     long long per_split = (long long)m * n * sizeof(float);
     if (splits > 1 && (long long)splits * per_split > workspace_bytes)
@@ -451,8 +498,9 @@ ROCML_EXPORT int rocml_gemm_residual_prescale_pays(int m, int n, int k) {
     return k <= 12288 && m <= 8 && 10 * tiles >= 9 * cus;
 }
 
-// algo: 0 = choose, 1 = plain tiled kernel, 2 = MFMA tile kernel, 3 = MFMA few-rows kernel (M <= 64),
-// 4 = MFMA kernel for at most 16 rows, 5 = MFMA tile kernel with 256x256 tiles.
+// algo: 0 = choose, 1 = plain tiled kernel, 2 = MFMA tile kernel (128x128 tiles), 3 = MFMA few-rows
+// kernel (M <= 64), 4 = MFMA kernel for at most 16 rows, 5 to 9 = MFMA tile kernel with 256x256,
+// 256x192, 128x192, 256x96 and 64x256 tiles.
 // accumulate: out += product (out must be 32-bit); this is the residual sum's epilogue.
 // epilogue: 0 = none; 1 = gated activation: W's rows are (gate_j, up_j) pairs and out is
 //   [M, N/2] = silu(gate) * up.
@@ -464,11 +512,13 @@ ROCML_EXPORT int rocml_gemm_residual_prescale_pays(int m, int n, int k) {
 //   come: row_ssq[M][row_parts] are sums of squares of x whose total over a row gives the row's
 //   scale 1 / sqrt(total / K + row_eps), which the gated epilogue applies to its sums.  Only for
 //   the gated epilogue of at most 16 rows on the MFMA path.
+// max_splits: the most pieces K may be cut into (0: the kernels' own limit of 16), for a caller
+//   whose next kernel adds a few partial sums cheaply and more of them one after the other.
 ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, int w_dtype, int ldw,
                             void* out, int out_dtype, int ldo, int m, int n, int k, int accumulate,
                             int algo, int epilogue, int defer, int* deferred_splits, void* workspace,
                             long long workspace_bytes, const float* row_ssq, int row_parts, float row_eps,
-                            hipStream_t stream) {
+                            int max_splits, hipStream_t stream) {
     if (deferred_splits) *deferred_splits = 0;
     ROCML_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm: bad sizes M=%d N=%d K=%d", m, n, k);
     bool gated = epilogue == 1;
@@ -478,7 +528,7 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
     ROCML_REQUIRE(ldx >= k && ldw >= k && ldo >= out_cols, "gemm: row strides (%d, %d, %d) below (K, K, N)",
                   ldx, ldw, ldo);
     ROCML_REQUIRE(!accumulate || out_dtype == ROCML_F32, "gemm: accumulation needs a 32-bit output");
-    ROCML_REQUIRE(algo >= ALGO_AUTO && algo <= ALGO_MFMA_TILE192, "gemm: unknown algorithm %d", algo);
+    ROCML_REQUIRE(algo >= ALGO_AUTO && algo <= ALGO_MFMA_TILE64X256, "gemm: unknown algorithm %d", algo);
     ROCML_REQUIRE(!defer || deferred_splits, "gemm: deferring needs a place to report the splits");
     if (m == 0) return 0;
     bool bf16_in = x_dtype == ROCML_BF16 && w_dtype == ROCML_BF16;
@@ -508,7 +558,8 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
         const int cus = cu_count();
         bool few_rows = m <= 16 || (m <= 64 && (gated || (m <= 48 && n < 256 * cus)));
         bool skinny = algo == ALGO_MFMA_SKINNY || (algo == ALGO_AUTO && few_rows);
-        SplitPlan plan{defer, deferred_splits, RowScale{row_ssq, row_parts, row_eps, 1.0f / (float)k}};
+        SplitPlan plan{defer, deferred_splits, RowScale{row_ssq, row_parts, row_eps, 1.0f / (float)k},
+                       max_splits >= 1 && max_splits < 16 ? max_splits : 16};
         int rc;
 #define BY_EPI(fn, ...)                                              \
         (epi == EPI_F32 ? fn<EPI_F32>(__VA_ARGS__)                   \
@@ -525,7 +576,9 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
         if (kpar) rc = BY_EPI(launch_kpar, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
         else if (skinny) rc = BY_EPI(launch_skinny_m, x, ldx, w, ldw, out, ldo, m, n, k, workspace, workspace_bytes, plan, stream);
         else rc = BY_EPI(launch_mfma_tile, x, ldx, w, ldw, out, ldo, m, n, k,
-                         algo == ALGO_MFMA_TILE ? 1 : algo == ALGO_MFMA_TILE256 ? 2 : algo == ALGO_MFMA_TILE192 ? 3 : 0,
+                         algo == ALGO_MFMA_TILE ? 1 : algo == ALGO_MFMA_TILE256 ? 2 : algo == ALGO_MFMA_TILE192 ? 3
+                         : algo == ALGO_MFMA_TILE128X192 ? 4 : algo == ALGO_MFMA_TILE256X96 ? 5
+                         : algo == ALGO_MFMA_TILE64X256 ? 6 : 0,
                          workspace, workspace_bytes,
                          plan, stream);
 #undef BY_EPI

@@ -36,7 +36,7 @@ _SIGNATURES = {
         "rocml_add_into": [_P, _P, _I, _LL, _P],
     },
     "gemm": {
-        "rocml_gemm": [_P, _I, _I, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _LL, _P, _I, _F, _P],
+        "rocml_gemm": [_P, _I, _I, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _LL, _P, _I, _F, _I, _P],
         "rocml_splitk_reduce": [_P, _P, _I, _I, _I, _I, _I, _I, _P],
         "rocml_gemm_residual_prescale_pays": [_I, _I, _I],
         "rocml_gemm_residual_prescale": [_P, _I, _P, _I, _P, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P],
@@ -295,14 +295,15 @@ class RowScale:
 
 def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
          algo: int = GEMM_AUTO, workspace: Optional[torch.Tensor] = None, epilogue: Optional[str] = None,
-         defer: bool = False, row_scale: Optional["RowScale"] = None) -> int:
+         defer: bool = False, row_scale: Optional["RowScale"] = None, max_splits: int = 0) -> int:
     """``out (+)= x @ w.T`` for ``x [M, K]``, ``w [N, K]``, ``out [M, N]`` (rows may be
     strided views with unit inner stride).  ``epilogue="swiglu"``: ``w``'s rows are (gate, up)
     pairs and ``out`` is ``[M, N/2] = silu(gate) * up``.  With ``defer`` a product that was
     split along K leaves its partial sums ``[splits, M, N]`` at the start of ``workspace`` and
     returns their number for the caller's next kernel to add; it returns 0 when ``out`` is
     complete.  ``row_scale``: ``x`` lacks its norm's scale (see ``RowScale``), which the gated
-    epilogue applies; at most ``ROW_SCALE_MAX_ROWS`` rows."""
+    epilogue applies; at most ``ROW_SCALE_MAX_ROWS`` rows.  ``max_splits``: the most pieces K may
+    be cut into (0: as the kernels see fit)."""
     for t in (x, w, out):
         if not t.is_cuda:
             raise KernelError("kernel arguments must be GPU tensors; this library has no CPU path")
@@ -326,7 +327,7 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         _ptr(x), _code(x), x.stride(0) if m > 1 else max(x.stride(0), k), _ptr(w), _code(w), w.stride(0),
         _ptr(out), _code(out), out.stride(0) if m > 1 else max(out.stride(0), cols), m, n, k,
         1 if accumulate else 0, algo, 1 if epilogue else 0, 1 if defer else 0, ctypes.byref(deferred), ws_ptr,
-        ws_bytes, ssq_ptr, parts, eps, _stream()))
+        ws_bytes, ssq_ptr, parts, eps, int(max_splits), _stream()))
     return deferred.value
 
 
@@ -433,6 +434,11 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache
 
 FUSED_DECODE_HEAD_DIMS = (64, 128, 192, 256)
 FUSED_DECODE_PAGE = 64
+# The most partial sums of the projection the fused decode attention should be handed: it adds four in
+# one trip to memory and each further one in a trip of its own.  Measured at 64 sequences (8B shape,
+# decoded tokens a second): at most 4 pieces 8,022, 5 8,073, 6 8,003, 8 7,932, no limit 7,960; at 16
+# to 48 sequences the limit makes no difference.
+FUSED_DECODE_SPLITS = 5
 
 
 def decode_splits(pairs: int, n_cus: int, most: int) -> int:

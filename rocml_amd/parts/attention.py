@@ -117,7 +117,10 @@ class Attention(Mixer):
         rows = self.q_dim + 2 * self.kv_dim if owns_cache else self.q_dim
         qkv = ws.get("attn.qkv", (n, rows), torch.float32)
         scratch = ws.scratch()
-        splits = ops.gemm(xn, self.w_qkv[:rows], qkv, workspace=scratch, defer=True)
+        # (the decode kernel that reads the projection adds four partial sums in one trip to memory
+        # and further ones one after the other: K is cut into few pieces for it)
+        splits = ops.gemm(xn, self.w_qkv[:rows], qkv, workspace=scratch, defer=True,
+                          max_splits=ops.FUSED_DECODE_SPLITS if self._fused_decode(step) else 0)
         if splits:      # the product's split-K partial sums; the next kernel adds them
             qkv = scratch[:splits * n * rows * 4].view(torch.float32).view(splits, n, rows)
         cos = sin = None

@@ -9,7 +9,7 @@ pytestmark = pytest.mark.gpu
 from rocml_amd import ops  # noqa: E402
 from rocml_amd.errors import KernelError  # noqa: E402
 
-PLAIN, TILE, SKINNY, KPAR, TILE256, TILE192 = 1, 2, 3, 4, 5, 6
+PLAIN, TILE, SKINNY, KPAR, TILE256, TILE192, TILE128X192, TILE256X96, TILE64X256 = 1, 2, 3, 4, 5, 6, 7, 8, 9
 
 
 def _operands(m, n, k, dtype, seed):
@@ -40,7 +40,7 @@ SHAPES = [(1, 64, 64), (5, 200, 72), (16, 130, 512), (17, 96, 264), (33, 4096, 1
           (8, 1000, 2056), (128, 128, 64), (129, 300, 200), (300, 515, 72), (2048, 512, 1024)]
 
 
-@pytest.mark.parametrize("algo", [PLAIN, TILE, SKINNY, KPAR, TILE256, TILE192])
+@pytest.mark.parametrize("algo", [PLAIN, TILE, SKINNY, KPAR, TILE256, TILE192, TILE128X192, TILE256X96, TILE64X256])
 @pytest.mark.parametrize("m,n,k", SHAPES)
 def test_bfloat16_algorithms(m, n, k, algo):
     if (algo == SKINNY and m > 64) or (algo == KPAR and m > 16):
@@ -80,7 +80,7 @@ def test_strided_rows_and_refusals():
         ops.gemm(x.cpu(), w, out)
 
 
-@pytest.mark.parametrize("algo", [PLAIN, TILE, SKINNY, KPAR, TILE256, TILE192])
+@pytest.mark.parametrize("algo", [PLAIN, TILE, SKINNY, KPAR, TILE256, TILE192, TILE128X192, TILE256X96, TILE64X256])
 @pytest.mark.parametrize("m,n,k", [(1, 64, 64), (7, 448, 96), (25, 300, 520), (41, 130, 1032), (64, 1000, 264), (130, 256, 128), (300, 2048, 512)])
 def test_gated_epilogue(m, n, k, algo):
     """Rows of the weight are (gate, up) pairs; the output is silu(gate) * up, formed from
