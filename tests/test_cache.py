@@ -292,3 +292,23 @@ def test_a_request_class_derived_from_a_registered_one_gets_its_own_group():
     assert _group_type(PlainChild(1, 16)) is KVGroup and _group_type(KVCacheRequest(1, 16)) is KVGroup
     c = Cache([WideRequest(1, 16), KVCacheRequest(1, 16)], max_tokens=128, dtype=torch.float32, device="cpu")
     assert type(c.line(0)[0]) is WideGroup and type(c.line(1)[0]) is KVGroup
+
+
+def test_workspace_views_are_kept_until_their_buffer_moves():
+    """A step asks for the same few views over and over; the workspace hands the same view out
+    again, and forgets a buffer's views when the buffer has to grow (a recorded graph is then
+    stale, which ``generation`` says)."""
+    from rocml_amd.engine import Workspace
+    ws = Workspace("cpu")
+    a = ws.get("x", (4, 8), torch.float32)
+    g0 = ws.generation
+    assert ws.get("x", (4, 8), torch.float32) is a and ws.generation == g0
+    b = ws.get("x", (2, 8), torch.float32)                    # a smaller view of the same buffer
+    assert b.data_ptr() == a.data_ptr() and ws.generation == g0 and tuple(b.shape) == (2, 8)
+    other = ws.get("x", (4, 8), torch.bfloat16)               # another type is another buffer
+    assert other.dtype == torch.bfloat16 and ws.generation == g0 + 1
+    big = ws.get("x", (16, 8), torch.float32)                 # the buffer grows: its views are dropped
+    assert ws.generation == g0 + 2 and tuple(big.shape) == (16, 8)
+    again = ws.get("x", (4, 8), torch.float32)
+    assert again is not a and again.data_ptr() == big.data_ptr()
+    assert ws.get("x", (4, 8), torch.bfloat16) is other       # the other buffer's views stay
