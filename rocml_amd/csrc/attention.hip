@@ -64,12 +64,15 @@ static int launch_decode(const AttnArgs& a, hipStream_t stream) {
     if (n_splits < 1) n_splits = 1;
     float* part_o = (float*)a.workspace;
     float* part_ml = part_o ? part_o + (size_t)a.n_tokens * a.hq * n_splits * D : nullptr;
-    // Many splits mean few pieces per block: then two of a wave's pieces travel at a time.  The
-    // choice follows the launch's shape, not the lengths, as the number of splits does.
+    // Many splits mean few pieces per block: then two of a wave's pieces travel at a time; so they
+    // do when the chip holds at most one block a CU (a long loop then gains from it what a second
+    // block would bring).  The choice follows the launch's shape, not the lengths, as the number of
+    // splits does.
     int rc;
     if constexpr (D <= 128)
-        rc = n_splits >= 4 ? launch_decode_kernel<D, FUSED, 2>(a, n_splits, part_o, part_ml, stream)
-                           : launch_decode_kernel<D, FUSED, 1>(a, n_splits, part_o, part_ml, stream);
+        rc = n_splits >= 4 || (long long)a.n_tokens * a.hkv * n_splits <= cu_count()
+                 ? launch_decode_kernel<D, FUSED, 2>(a, n_splits, part_o, part_ml, stream)
+                 : launch_decode_kernel<D, FUSED, 1>(a, n_splits, part_o, part_ml, stream);
     else
         rc = launch_decode_kernel<D, FUSED, 1>(a, n_splits, part_o, part_ml, stream);
     if (rc) return rc;
