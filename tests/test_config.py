@@ -101,11 +101,11 @@ def test_catalog_and_resolve(tmp_path):
 
 
 def test_decode_splits_fill_the_chip_evenly():
-    """Key-range splits of a decode step: about two blocks a CU for a few sequences; from eight
+    """Key-range splits of a decode step: about a block a CU for a few sequences; from eight
     sequences' worth of (token, kv head) pairs on, the count that leaves the busiest CU the least
     work when every block and every merge has a fixed price; never more than the pages there are."""
     from rocml_amd.ops import decode_splits
-    assert [decode_splits(b * 8, 256, 64) for b in (1, 2, 4, 8, 16, 32, 64, 128)] == [64, 32, 16, 4, 2, 1, 1, 1]
+    assert [decode_splits(b * 8, 256, 64) for b in (1, 2, 4, 8, 16, 32, 64, 128)] == [32, 16, 8, 4, 2, 1, 1, 1]
     assert decode_splits(24 * 8, 256, 64) == 1          # 192 blocks, one a CU with two pieces on their way, no merge
     assert decode_splits(14 * 8, 256, 64) == 2          # not 9: 1,008 tiny blocks and a merge of nine
     assert decode_splits(18 * 8, 256, 64) == 3          # 432 blocks, under two a CU
