@@ -186,6 +186,7 @@ __device__ __forceinline__ void epilogue_store(void* out, size_t idx, float v) {
 // and the compiler answers such loads with a full wait on the LDS counter before the first
 // product of every stage.)
 constexpr int GM_BK = 64;
+constexpr int GM_BAND = 8;                             // tile rows of a band (see the kernel)
 constexpr int GM_ROW = GM_BK / 8 + 1;                 // u32x4_t per LDS row, one of padding
 
 template <int WAVES_M_, int WAVES_N_, int TM_, int TN_>
@@ -266,7 +267,12 @@ gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
     x += ks;
     w += ks;
     out = (float*)out + split * split_stride;
-    int m0 = (logical % tiles_m) * T::BM, n0 = (logical / tiles_m) * T::BN;
+    // Tiles are walked in bands of eight tile rows, down the band's columns: the 32 blocks that an
+    // XCD holds at a time are then eight tile rows by four tile columns (twelve operand strips
+    // through its L2 for 32 tiles) and not 32 rows of one column (33 strips), whatever the number of rows.
+    int band_tiles = GM_BAND * (n_tiles / tiles_m), band = logical / band_tiles, in_band = logical - band * band_tiles;
+    int band_rows = min(GM_BAND, tiles_m - band * GM_BAND);
+    int m0 = (band * GM_BAND + in_band % band_rows) * T::BM, n0 = (in_band / band_rows) * T::BN;
     int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     int wm = wave / T::WAVES_N, wn = wave % T::WAVES_N;
     int lrow = tid >> 3, lkc = tid & 7;

@@ -37,7 +37,8 @@ def test_plain_float32(m, n, k):
 
 
 SHAPES = [(1, 64, 64), (5, 200, 72), (16, 130, 512), (17, 96, 264), (33, 4096, 1024), (48, 1000, 776), (64, 257, 4096),
-          (8, 1000, 2056), (128, 128, 64), (129, 300, 200), (300, 515, 72), (2048, 512, 1024)]
+          (8, 1000, 2056), (128, 128, 64), (129, 300, 200), (300, 515, 72), (2048, 512, 1024),
+          (1409, 300, 128), (2561, 200, 64)]       # 12 and 21 tile rows of 128, 6 and 11 of 256: whole bands of eight and a rest
 
 
 @pytest.mark.parametrize("algo", [PLAIN, TILE, SKINNY, KPAR, TILE256, TILE192, TILE128X192, TILE256X96, TILE64X256])
