@@ -417,6 +417,7 @@ __global__ void attn_decode_reduce_kernel(const float* __restrict__ part_o, cons
 // keys and values go through LDS once per block; every wave multiplies its 32 queries with them.
 constexpr int AM_ROUND = 256;                           // blocks that start together: one per CU
 constexpr int AM_QTILE = 128;                           // query rows of a block: 32 per wave
+constexpr float AM_LAZY_MAX = 8.0f;                     // how far a row's maximum may run ahead of its exponents' reference
 
 template <int D>
 struct PrefillLds {
@@ -574,19 +575,15 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
 #pragma unroll
             for (int e = 1; e < 16; ++e) mx = fmaxf(mx, s[e]);
             mx = max_across_halves(mx) * scale_log2e;       // the scale is positive
-            float m_new = fmaxf(m, mx);
-            float m_use = m_new == -INFINITY ? 0.f : m_new;
-            float sum = 0.f;
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                s[e] = fast_exp2(fmaf(s[e], scale_log2e, -m_use));
-                sum += s[e];
-            }
-            sum = sum_across_halves(sum);
-            // the running maximum rarely moves after the first pieces: rescale only when some
-            // row of the wave needs it
-            if (__builtin_amdgcn_ballot_w64(m_new != m)) {
-                float corr = fast_exp2(m - m_use);
+            // The exponents' reference m follows a row's maximum only when that has grown by more
+            // than AM_LAZY_MAX (powers of two): any reference gives the same quotient at the end,
+            // the probabilities stay below 2^AM_LAZY_MAX, which bfloat16 and the 32-bit sums hold
+            // with room to spare, and the sums and outputs so far have to be rescaled (64 products
+            // a lane) only for the first pieces of a row instead of whenever one of a wave's 32
+            // rows meets a new maximum, which with a thousand keys behind it is still every other piece.
+            if (__builtin_amdgcn_ballot_w64(mx > m + AM_LAZY_MAX)) {
+                float m_new = fmaxf(m, mx);
+                float corr = fast_exp2(m - (m_new == -INFINITY ? 0.f : m_new));
                 l *= corr;
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
@@ -594,6 +591,14 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                     for (int e = 0; e < 16; ++e) o[dt][e] *= corr;
                 m = m_new;
             }
+            float m_use = m == -INFINITY ? 0.f : m;
+            float sum = 0.f;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                s[e] = fast_exp2(fmaf(s[e], scale_log2e, -m_use));
+                sum += s[e];
+            }
+            sum = sum_across_halves(sum);
             l += sum;
             // P^T operands: MFMA u takes elements 8u..8u+7 = keys 16u + {4 h2 .. +3, 8 + 4 h2 .. +3}.
             bf16x8_t pf[2];

@@ -387,6 +387,35 @@ def _long_case(length, n_new, hq, hkv, d, window, n_splits, seed):
     assert float((ref[0, 0] - vs[0][:length - n_new, 0].double().mean(0)).abs().max()) > 0.1
 
 
+@pytest.mark.parametrize("climb", [30.0, 4.0, -30.0])
+def test_prompt_whose_scores_climb_slowly(climb):
+    """The prefill kernel moves the reference of a row's exponents only when the row's maximum has
+    run ahead of it by more than 2^8.  Keys that lie along the queries of a kv head's first query
+    head, a little longer from one position to the next: the maximum grows by less than that per
+    piece for many pieces (probabilities far above one in between) and by several times that over
+    the sequence; with ``climb`` = 4 it never moves again after the first piece; falling scores
+    never move it at all.  Every row against the 64-bit softmax."""
+    hq, hkv, d, length, n_new = 4, 2, 128, 1500, 300
+    seqs = [(length, n_new)]
+    dev, ks, vs, qs = _build(seqs, hq, hkv, d, torch.bfloat16, 41)
+    group = hq // hkv
+    k, q, table = ks[0], qs[0], dev["table"].cpu()
+    scale = 1.0 / math.sqrt(d)
+    for j in range(hkv):
+        lead = torch.randn(d, generator=torch.Generator().manual_seed(50 + j))
+        lead = lead / lead.norm()
+        q[:, j * group] = (lead * math.sqrt(d)).to(torch.bfloat16)          # score of key p: its length along lead
+        ramp = torch.arange(length, dtype=torch.float32) / length * climb
+        k[:, j] = (ramp[:, None] * lead[None, :] + 0.05 * k[:, j].float()).to(torch.bfloat16)
+    dev["q"] = q.reshape(-1, hq * d).cuda()
+    for p_ in range(length):
+        dev["kc"][int(table[0, p_ // PAGE]), :, p_ % PAGE] = k[p_].cuda()
+    got = _run(dev, seqs, hq, hkv, d, scale, None, MFMA).double().reshape(-1, hq, d)
+    ref = _reference_rows(q, k, vs[0], list(range(length - n_new, length)), scale, None)
+    err = float((got - ref).abs().max())
+    assert err < 1.5e-2, f"climb {climb}: error {err}"
+
+
 @pytest.mark.parametrize("length", [32768, 40960])
 @pytest.mark.parametrize("window,n_splits", [(None, 1), (None, 8), (None, 64), (None, 0), (4096, 8), (4096, 64), (70, 0)])
 def test_decode_over_tens_of_thousands_of_keys(length, window, n_splits):
