@@ -28,6 +28,7 @@ struct AttnArgs {
     int hq, hkv; float scale; int window; void* workspace; long long workspace_bytes;
     int n_splits_hint;
     const DecodeProj* proj;     // decode only: the step's q/k/v projection instead of q and an appended cache
+    const PrefillProj* prefill_proj = nullptr;      // prompts: the projection instead of prepared queries
 };
 
 template <int D, bool FUSED, int AHEAD>
@@ -89,13 +90,19 @@ template <int D>
 static int launch_prefill(const AttnArgs& a, hipStream_t stream) {
     static bool ready = false;
     if (!ready) {
-        if (allow_lds(attn_prefill_mfma_kernel<D>, PrefillLds<D>::BYTES)) return 1;
+        if (allow_lds(attn_prefill_mfma_kernel<D, false>, PrefillLds<D>::BYTES)) return 1;
+        if (allow_lds(attn_prefill_mfma_kernel<D, true>, PrefillLds<D>::BYTES)) return 1;
         ready = true;
     }
     dim3 grid(a.total_q_tiles * a.hq);
-    attn_prefill_mfma_kernel<D><<<grid, AM_THREADS, PrefillLds<D>::BYTES, stream>>>(
-        a.q, a.out, a.kcache, a.vcache, a.block_table, a.bt_width, a.cu_seqlens, a.n_seqs, a.token_pos,
-        a.hq, a.hkv, a.scale * LOG2E, a.window);
+    if (a.prefill_proj)
+        attn_prefill_mfma_kernel<D, true><<<grid, AM_THREADS, PrefillLds<D>::BYTES, stream>>>(
+            nullptr, a.out, a.kcache, a.vcache, a.block_table, a.bt_width, a.cu_seqlens, a.n_seqs, a.token_pos,
+            a.hq, a.hkv, a.scale * LOG2E, a.window, *a.prefill_proj);
+    else
+        attn_prefill_mfma_kernel<D, false><<<grid, AM_THREADS, PrefillLds<D>::BYTES, stream>>>(
+            a.q, a.out, a.kcache, a.vcache, a.block_table, a.bt_width, a.cu_seqlens, a.n_seqs, a.token_pos,
+            a.hq, a.hkv, a.scale * LOG2E, a.window, PrefillProj{});
     return 0;
 }
 
@@ -220,5 +227,54 @@ ROCML_EXPORT int rocml_attention_decode_fused(const float* qkv, int ld, int qkv_
              : d == 192 ? launch_decode_fused<192>(a, stream) : launch_decode_fused<256>(a, stream);
     if (rc) return rc;
     ROCML_CHECK_LAUNCH("fused decode attention");
+    return 0;
+}
+
+// Prompts: attention of a step's new tokens over the cache, with the queries taken from the step's
+// q/k/v projection (32-bit, complete sums: a token's q heads first) and prepared by the kernel
+// itself: per-head norm (q_gain null: none), rotation of the whole head with pairs (e, e + D/2)
+// (cos/sin null: none, else [tokens, D/2]), rounding to bfloat16.  The keys and values of the new
+// tokens are in the cache already.  bfloat16 caches with pages of 64 positions and the MFMA
+// kernels' head sizes; cu_seqlens, q_counts as in rocml_attention.
+ROCML_EXPORT int rocml_attention_prefill_fused(const float* qkv, int ld, const float* q_gain, float eps,
+                                               const float* cos_t, const float* sin_t, void* out,
+                                               const void* kcache, const void* vcache, const int* block_table,
+                                               int bt_width, const int* token_pos, int n_tokens, int hq, int hkv,
+                                               int d, int page_size, float scale, int window,
+                                               const int* cu_seqlens, int n_seqs, const int* q_counts,
+                                               hipStream_t stream) {
+    ROCML_REQUIRE(n_tokens >= 0 && hq > 0 && hkv > 0 && bt_width > 0 && n_seqs > 0 && cu_seqlens && q_counts,
+                  "fused prefill attention: bad sizes T=%d Hq=%d Hkv=%d width=%d sequences=%d", n_tokens, hq, hkv,
+                  bt_width, n_seqs);
+    ROCML_REQUIRE(hq % hkv == 0, "fused prefill attention: %d query heads are not a multiple of %d kv heads", hq, hkv);
+    ROCML_REQUIRE(page_size == AM_PAGE && mfma_head_dim(d),
+                  "fused prefill attention: needs pages of 64 positions and a head size of 32, 64, 96, 128, 192 or 256 "
+                  "(page=%d D=%d)", page_size, d);
+    ROCML_REQUIRE(window >= 0, "fused prefill attention: negative window %d", window);
+    ROCML_REQUIRE(ld >= hq * d && ld % 4 == 0 && ((uintptr_t)qkv & 15) == 0,
+                  "fused prefill attention: projection rows of %d values (need %d, a multiple of 4, 16-byte aligned)",
+                  ld, hq * d);
+    ROCML_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "fused prefill attention: rotation tables come in pairs");
+    ROCML_REQUIRE(!q_gain || ((uintptr_t)q_gain & 15) == 0, "fused prefill attention: the gain must be 16-byte aligned");
+    ROCML_REQUIRE(!cos_t || ((((uintptr_t)cos_t | (uintptr_t)sin_t) & 15) == 0),
+                  "fused prefill attention: the rotation tables must be 16-byte aligned");
+    if (n_tokens == 0) return 0;
+    long long total_q_tiles = 0, counted = 0;
+    for (int b = 0; b < n_seqs; ++b) {
+        ROCML_REQUIRE(q_counts[b] >= 0, "fused prefill attention: sequence %d has %d query tokens", b, q_counts[b]);
+        total_q_tiles += (q_counts[b] + AM_QTILE - 1) / AM_QTILE;
+        counted += q_counts[b];
+    }
+    ROCML_REQUIRE(counted == n_tokens, "fused prefill attention: the sequences' query counts add up to %lld, the step has %d tokens",
+                  counted, n_tokens);
+    ROCML_REQUIRE(total_q_tiles > 0 && total_q_tiles * hq < (1ll << 31), "fused prefill attention: %lld query tiles", total_q_tiles);
+    PrefillProj pj{qkv, ld, q_gain, eps, cos_t, sin_t};
+    AttnArgs a{nullptr, (bf16_t*)out, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table, bt_width,
+               nullptr, token_pos, cu_seqlens, n_seqs, n_tokens, (int)total_q_tiles, 0, hq, hkv, scale, window, nullptr,
+               0, 0, nullptr};
+    a.prefill_proj = &pj;
+    int rc = BY_HEAD_DIM(launch_prefill, d, a, stream);
+    if (rc) return rc;
+    ROCML_CHECK_LAUNCH("fused prefill attention");
     return 0;
 }

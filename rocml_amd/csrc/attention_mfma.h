@@ -426,14 +426,24 @@ struct PrefillLds {
     static constexpr int BYTES = (AM_PAGE * K_ROW + D * V_ROW) * 2;
 };
 
-template <int D>
+// QPREP: the queries come as the step's q/k/v projection (32-bit, complete sums) and are
+// prepared here, per-head norm, rotation of the whole head with pairs (e, e + D/2) and rounding,
+// as the norm-and-rotation kernel would have prepared them; that kernel then only appends keys and
+// values, and the queries are neither written nor read as bfloat16 in between.
+struct PrefillProj {
+    const float* qkv; int ld;                           // [T, ld]: a token's q heads first
+    const float* q_gain; float eps;                     // null: no norm
+    const float* cos_t; const float* sin_t;             // [T, D/2], null: no rotation
+};
+
+template <int D, bool QPREP>
 __global__ void __launch_bounds__(AM_THREADS, D <= 128 ? 2 : 1)
 attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                          const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
                          const int* __restrict__ block_table, int bt_width,
                          const int* __restrict__ cu_seqlens, int n_seqs,
                          const int* __restrict__ token_pos, int hq, int hkv, float scale_log2e,
-                         int window) {
+                         int window, PrefillProj pj) {
     using L = PrefillLds<D>;
     constexpr int KK = D / 16;      // MFMA steps along D for the scores
     constexpr int DT = D / 32;      // 32-row tiles of the output
@@ -478,7 +488,58 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
 
     // Q^T operand: column = query row, 8 values of D per lane and step.
     bf16x8_t qf[KK];
-    {
+    if constexpr (QPREP) {
+        // this lane's 8 values of every 16 of its row; the other 8 are in the lane 32 away
+        int t = tok0 + (row_ok ? my_row : 0);
+        const float* qrow = pj.qkv + (size_t)t * pj.ld + (size_t)h * D + h2 * 8;
+        float qv[KK][8];
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            float4 lo = *(const float4*)(qrow + kk * 16), hi = *(const float4*)(qrow + kk * 16 + 4);
+            qv[kk][0] = lo.x; qv[kk][1] = lo.y; qv[kk][2] = lo.z; qv[kk][3] = lo.w;
+            qv[kk][4] = hi.x; qv[kk][5] = hi.y; qv[kk][6] = hi.z; qv[kk][7] = hi.w;
+        }
+        if (pj.q_gain) {
+            float ss = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) ss = fmaf(qv[kk][i], qv[kk][i], ss);
+            ss += __shfl_xor(ss, 32, 64);
+            float inv = 1.0f / sqrtf(ss / (float)D + pj.eps);
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) {
+                const float* g = pj.q_gain + kk * 16 + h2 * 8;
+                float4 g0 = *(const float4*)g, g1 = *(const float4*)(g + 4);
+                qv[kk][0] *= inv * g0.x; qv[kk][1] *= inv * g0.y; qv[kk][2] *= inv * g0.z; qv[kk][3] *= inv * g0.w;
+                qv[kk][4] *= inv * g1.x; qv[kk][5] *= inv * g1.y; qv[kk][6] *= inv * g1.z; qv[kk][7] *= inv * g1.w;
+            }
+        }
+        if (pj.cos_t) {
+            // value e of the first half of the head and value e + D/2 are a pair: steps kk and kk + KK/2
+            const float* c = pj.cos_t + (size_t)t * (D / 2) + h2 * 8;
+            const float* sn = pj.sin_t + (size_t)t * (D / 2) + h2 * 8;
+#pragma unroll
+            for (int kk = 0; kk < KK / 2; ++kk) {
+                float cs[8], si[8];
+                *(float4*)cs = *(const float4*)(c + kk * 16); *(float4*)(cs + 4) = *(const float4*)(c + kk * 16 + 4);
+                *(float4*)si = *(const float4*)(sn + kk * 16); *(float4*)(si + 4) = *(const float4*)(sn + kk * 16 + 4);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    float lo = qv[kk][i], hi = qv[kk + KK / 2][i];
+                    qv[kk][i] = lo * cs[i] - hi * si[i];
+                    qv[kk + KK / 2][i] = lo * si[i] + hi * cs[i];
+                }
+            }
+        }
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            uint4 v = make_uint4(pack_bf16x2(qv[kk][0], qv[kk][1]), pack_bf16x2(qv[kk][2], qv[kk][3]),
+                                 pack_bf16x2(qv[kk][4], qv[kk][5]), pack_bf16x2(qv[kk][6], qv[kk][7]));
+            v.x = row_ok ? v.x : 0u; v.y = row_ok ? v.y : 0u; v.z = row_ok ? v.z : 0u; v.w = row_ok ? v.w : 0u;
+            qf[kk] = __builtin_bit_cast(bf16x8_t, v);
+        }
+    } else {
         const bf16_t* qrow = q + ((size_t)(tok0 + (row_ok ? my_row : 0)) * hq + h) * D + h2 * 8;
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {

@@ -285,14 +285,14 @@ __global__ void qk_norm_rope_append_kernel(
     TO* __restrict__ q_out, TO* __restrict__ kcache, TO* __restrict__ vcache,
     const int* __restrict__ block_table, int bt_width, const int* __restrict__ token_seq,
     const int* __restrict__ token_pos, int page_size, int write_kv, int n_splits, long long split_stride,
-    int rows_per_token, int pairing) {
+    int rows_per_token, int pairing, int first_row) {
     extern __shared__ float stage[];   // [QK_WAVES][d]
     int wave = threadIdx.x / WAVE;
     int lane = threadIdx.x & (WAVE - 1);
     long long row = (long long)blockIdx.x * QK_WAVES + wave;
     bool active = row < (long long)n_tokens * rows_per_token;
     int t = active ? (int)(row / rows_per_token) : 0;
-    int r = active ? (int)(row - (long long)t * rows_per_token) : 0;
+    int r = first_row + (active ? (int)(row - (long long)t * rows_per_token) : 0);     // first_row = hq: no q rows
     int kind = r < hq ? 0 : (r < hq + hkv ? 1 : 2);   // q, k, v
     if (!write_kv && kind != 0) active = false;
     const TI* src = qkv + (size_t)t * ld + (size_t)r * d;
@@ -412,7 +412,8 @@ qk_norm_rope_rows_kernel(
     const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     TO* __restrict__ q_out, TO* __restrict__ kcache, const int* __restrict__ block_table, int bt_width,
-    const int* __restrict__ token_seq, const int* __restrict__ token_pos, int page_size, int rows_per_token) {
+    const int* __restrict__ token_seq, const int* __restrict__ token_pos, int page_size, int rows_per_token,
+    int first_row) {
     constexpr int HJ = QK_PER_LANE / 2;
     int wave = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1);
     long long total = (long long)n_tokens * rows_per_token;
@@ -423,7 +424,7 @@ qk_norm_rope_rows_kernel(
     for (int i = 0; i < ROWS; ++i) {
         long long row = min(row0 + i, total - 1);            // rows past the end repeat the last one, not stored
         tok[i] = (int)(row / rows_per_token);
-        rr[i] = (int)(row - (long long)tok[i] * rows_per_token);
+        rr[i] = first_row + (int)(row - (long long)tok[i] * rows_per_token);
         const TI* src = qkv + (size_t)tok[i] * ld + (size_t)rr[i] * d;
 #pragma unroll
         for (int j = 0; j < QK_PER_LANE; ++j) v[i][j] = Elem<TI>::load(src + lane + j * WAVE);
@@ -526,10 +527,14 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     ROCML_REQUIRE(pairing == 0 || pairing == 1, "qk_norm_rope_append: pairing %d (0: halves, 1: neighbours)", pairing);
     ROCML_REQUIRE(!write_kv || (page_size > 0 && bt_width > 0 && block_table && kcache && vcache),
                   "qk_norm_rope_append: cache arguments missing");
+    ROCML_REQUIRE(q_out || write_kv, "qk_norm_rope_append: nothing to write");
     if (n_tokens == 0) return 0;
     // prompts: the values go through the transposing tile kernel, the row kernel does q and k
     bool v_tiled = write_kv && n_splits == 1 && n_tokens >= VT_TOKENS;
-    int rows_per_token = hq + (write_kv ? (v_tiled ? hkv : 2 * hkv) : 0);
+    // (without q_out the q rows are left to the caller: the prefill attention that reads the
+    // projection prepares its queries itself)
+    int first_row = q_out ? 0 : hq;
+    int rows_per_token = hq - first_row + (write_kv ? (v_tiled ? hkv : 2 * hkv) : 0);
     long long rows = (long long)n_tokens * rows_per_token;
     int per_lane = d <= 64 ? 1 : d <= 128 ? 2 : d <= 256 ? 4 : 8;     // head values per lane
     // both values of a rotation pair in one lane: whole head rotated, d = per_lane * 64
@@ -544,12 +549,12 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     qk_norm_rope_append_kernel<TI, TO, N, LP><<<grid, EW_BLOCK, lds, stream>>>(                 \
         (const TI*)qkv, ld, n_tokens, hq, hkv, d, q_gain, k_gain, eps, cos_t, sin_t, rot,       \
         (TO*)q_out, (TO*)kcache, (TO*)vcache, block_table, bt_width, token_seq, token_pos,      \
-        page_size, write_kv, n_splits, split_stride, rows_per_token, pairing)
+        page_size, write_kv, n_splits, split_stride, rows_per_token, pairing, first_row)
 #define LAUNCH_ROWS(TI, TO, N)                                                                  \
     qk_norm_rope_rows_kernel<TI, TO, N, MANY><<<grid, EW_BLOCK, 0, stream>>>(                   \
         (const TI*)qkv, ld, n_tokens, hq, hkv, d, q_gain, k_gain, eps, rot ? cos_t : nullptr,   \
         rot ? sin_t : nullptr, (TO*)q_out, (TO*)kcache, block_table, bt_width, token_seq,       \
-        token_pos, page_size, rows_per_token)
+        token_pos, page_size, rows_per_token, first_row)
 #define LAUNCH(TI, TO)                                                                          \
     {                                                                                           \
         if (many_rows) { if (per_lane == 2) LAUNCH_ROWS(TI, TO, 2); else LAUNCH_ROWS(TI, TO, 4); } \

@@ -46,6 +46,8 @@ _SIGNATURES = {
                             _P, _I, _I, _P, _I, _I, _P, _LL, _P],
         "rocml_attention_decode_fused": [_P, _I, _I, _LL, _P, _P, _F, _P, _P, _I, _P, _P, _P, _P, _I, _P, _P,
                                          _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _LL, _P, _I, _F, _I, _P],
+        "rocml_attention_prefill_fused": [_P, _I, _P, _F, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _I,
+                                          _P, _I, _P, _P],
     },
     "sampling": {
         "rocml_sample": [_P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _P],
@@ -218,7 +220,7 @@ ROPE_PAIRINGS = {"halves": 0, "neighbours": 1}
 def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,
                         q_gain: Optional[torch.Tensor], k_gain: Optional[torch.Tensor], eps: float,
                         cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rot_dim: int,
-                        q_out: torch.Tensor, k_cache: Optional[torch.Tensor],
+                        q_out: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
                         v_cache: Optional[torch.Tensor], block_table: Optional[torch.Tensor],
                         token_seq: torch.Tensor, token_pos: torch.Tensor, write_kv: bool = True,
                         n_splits: int = 1, pairing: str = "halves") -> None:
@@ -226,7 +228,8 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
     ``write_kv`` is false).  Keys are ``[pages, Hkv, page_size, D]``, values
     ``[pages, Hkv, D, page_size]``.  ``pairing``: which two values of the rotated width turn
     together by the angle in column ``i`` of the tables: ``"halves"``, ``(i, i + rot_dim / 2)``,
-    or ``"neighbours"``, ``(2 i, 2 i + 1)``."""
+    or ``"neighbours"``, ``(2 i, 2 i + 1)``.  ``q_out`` None: only keys and values are prepared
+    and appended (the caller's attention kernel prepares its queries itself)."""
     if pairing not in ROPE_PAIRINGS:
         raise KernelError(f"unknown rotation pairing {pairing!r}; known: {sorted(ROPE_PAIRINGS)}")
     _dev(qkv, q_gain, k_gain, cos, sin, q_out, k_cache, v_cache, block_table, token_seq, token_pos)
@@ -245,7 +248,9 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
     if cos is not None:
         if cos.shape != (n_tokens, rot_dim // 2) or sin is None or sin.shape != cos.shape:
             raise KernelError(f"rotation tables must be {(n_tokens, rot_dim // 2)}")
-    if q_out.shape != (n_tokens, n_heads * head_dim) or token_seq.numel() != n_tokens \
+    if q_out is None and not write_kv:
+        raise KernelError("nothing to do: no q output and no append to the cache")
+    if (q_out is not None and q_out.shape != (n_tokens, n_heads * head_dim)) or token_seq.numel() != n_tokens \
             or token_pos.numel() != n_tokens:
         raise KernelError("q output or token tables do not match the number of tokens")
     page_size = bt_width = 0
@@ -255,15 +260,15 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
         if k_cache.shape[1:] != (n_kv_heads, k_cache.shape[2], head_dim) \
                 or v_cache.shape != (k_cache.shape[0], n_kv_heads, head_dim, k_cache.shape[2]):
             raise KernelError(f"cache shape {tuple(k_cache.shape)} does not fit {n_kv_heads} heads of {head_dim}")
-        if k_cache.dtype != q_out.dtype:
+        if q_out is not None and k_cache.dtype != q_out.dtype:
             raise KernelError("cache and q output must share their type")
         _want(block_table, torch.int32, "block table")
         page_size, bt_width = k_cache.shape[2], block_table.shape[1]
     _check("elementwise", library("elementwise").rocml_qk_norm_rope_append(
         _ptr(qkv), _code(qkv), ld, n_tokens, n_heads, n_kv_heads, head_dim, _ptr(q_gain), _ptr(k_gain),
         eps, _ptr(cos), _ptr(sin), rot_dim if cos is not None else 0, ROPE_PAIRINGS[pairing], _ptr(q_out), _ptr(k_cache),
-        _ptr(v_cache), _code(q_out), _ptr(block_table), bt_width, _ptr(token_seq), _ptr(token_pos),
-        page_size, 1 if write_kv else 0, n_splits, split_stride, _stream()))
+        _ptr(v_cache), _code(q_out if q_out is not None else k_cache), _ptr(block_table), bt_width, _ptr(token_seq),
+        _ptr(token_pos), page_size, 1 if write_kv else 0, n_splits, split_stride, _stream()))
 
 
 def add_into(x: torch.Tensor, y: torch.Tensor) -> None:
@@ -476,6 +481,62 @@ def attention_decode_fusable(dtype: torch.dtype, n_heads: int, n_kv_heads: int, 
     whole head in pairs ``(i, i + head_dim / 2)``."""
     return (dtype == torch.bfloat16 and page == 64 and head_dim in FUSED_DECODE_HEAD_DIMS
             and n_heads // n_kv_heads <= 16 and (rot_dim is None or (rot_dim == head_dim and pairing == "halves")))
+
+
+PREFILL_FUSED_PAGE = 64
+PREFILL_FUSED_HEAD_DIMS = (32, 64, 96, 128, 192, 256)
+
+
+def attention_prefill_fusable(dtype: torch.dtype, head_dim: int, page_size: int, rot_dim: Optional[int],
+                              pairing: str = "halves") -> bool:
+    """Whether ``attention_prefill_fused`` takes a layer: a bfloat16 cache with pages of 64 positions,
+    a head size the MFMA kernels know, and a rotation of the whole head with halves as pairs (or none)."""
+    return (dtype == torch.bfloat16 and page_size == PREFILL_FUSED_PAGE and head_dim in PREFILL_FUSED_HEAD_DIMS
+            and (rot_dim is None or (rot_dim == head_dim and pairing == "halves")))
+
+
+def attention_prefill_fused(qkv: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                            block_table: torch.Tensor, token_pos: torch.Tensor, n_heads: int, n_kv_heads: int,
+                            head_dim: int, scale: float, q_gain: Optional[torch.Tensor], eps: float,
+                            cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], window: Optional[int],
+                            cu_seqlens: torch.Tensor, q_counts: Sequence[int]) -> None:
+    """A prompt step's attention with the queries taken from the q/k/v projection ``qkv`` (float32
+    ``[tokens, ld]``, complete sums, a token's q heads first): per-head norm, rotation and rounding
+    of the queries happen in the attention kernel.  The new tokens' keys and values are in the
+    cache already (``qk_norm_rope_append`` without a q output puts them there)."""
+    _dev(qkv, out, k_cache, v_cache, block_table, token_pos, q_gain, cos, sin, cu_seqlens)
+    _want(qkv, torch.float32, "projection output")
+    if qkv.dim() != 2:
+        raise KernelError("the projection must be [tokens, width] (complete sums)")
+    n_tokens, ld = qkv.shape
+    page = k_cache.shape[2]
+    if not attention_prefill_fusable(k_cache.dtype, head_dim, page, None if cos is None else 2 * cos.shape[-1]):
+        raise KernelError(f"fused prefill attention does not take this layer (cache {k_cache.dtype}, pages of {page}, "
+                          f"head size {head_dim})")
+    if out.shape != (n_tokens, n_heads * head_dim) or out.dtype != k_cache.dtype:
+        raise KernelError("attention output must be [tokens, heads * head_dim] of the cache's type")
+    if v_cache.dtype != k_cache.dtype or k_cache.shape[1:] != (n_kv_heads, page, head_dim) \
+            or v_cache.shape != (k_cache.shape[0], n_kv_heads, head_dim, page):
+        raise KernelError(f"cache {tuple(k_cache.shape)} / {tuple(v_cache.shape)} does not fit {n_kv_heads} heads of {head_dim}")
+    if q_gain is not None:
+        _want(q_gain, torch.float32, "head norm gain")
+        if q_gain.numel() != head_dim:
+            raise KernelError(f"head norm gain has {q_gain.numel()} values for head size {head_dim}")
+    if cos is not None:
+        _want(cos, torch.float32, "rotation table")
+        if cos.shape != (n_tokens, head_dim // 2) or sin is None or sin.shape != cos.shape or sin.dtype != cos.dtype:
+            raise KernelError(f"rotation tables must be float32 {(n_tokens, head_dim // 2)}")
+    _want(block_table, torch.int32, "block table")
+    _want(token_pos, torch.int32, "token position table")
+    _want(cu_seqlens, torch.int32, "sequence offsets")
+    n_seqs = cu_seqlens.numel() - 1
+    if token_pos.numel() != n_tokens or len(q_counts) != n_seqs or block_table.shape[0] < n_seqs:
+        raise KernelError("one position per token, one query count and one block table row per sequence are needed")
+    counts = (ctypes.c_int * n_seqs)(*[int(c) for c in q_counts])
+    _check("attention", library("attention").rocml_attention_prefill_fused(
+        _ptr(qkv), ld, _ptr(q_gain), eps, _ptr(cos), _ptr(sin), _ptr(out), _ptr(k_cache), _ptr(v_cache),
+        _ptr(block_table), block_table.shape[1], _ptr(token_pos), n_tokens, n_heads, n_kv_heads, head_dim, page,
+        scale, 0 if window is None else int(window), _ptr(cu_seqlens), n_seqs, counts, _stream()))
 
 
 def attention_decode_fused(qkv: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,

@@ -95,6 +95,11 @@ class Attention(Mixer):
         return step.max_new == 1 and ops.attention_decode_fusable(
             self.dtype, self.spec.n_heads, self.spec.n_kv_heads, self.spec.head_dim, ops.FUSED_DECODE_PAGE, rot, self.pairing)
 
+    def _fused_prefill(self, step, cache) -> bool:
+        rot = None if self.position is None else self.position.rot_dim
+        return (step.max_new > 1 and step.cu_seqlens is not None and self.dtype == torch.bfloat16
+                and ops.attention_prefill_fusable(cache.k.dtype, self.spec.head_dim, cache.k.shape[2], rot, self.pairing))
+
     def takes_row_scale(self, step) -> bool:
         # only the decode kernel that reads the projection's sums itself applies a scale to them
         return self._fused_decode(step)
@@ -143,14 +148,25 @@ class Attention(Mixer):
         else:
             if stream(step).row_scale is not None:
                 raise ConfigError("the attention was handed an input without its norm's scale in a step it cannot scale")
-            q = ws.get("attn.q", (n, self.q_dim), self.dtype)
-            ops.qk_norm_rope_append(qkv, s.n_heads, s.n_kv_heads, s.head_dim, self.q_gain, self.k_gain, eps,
-                                    cos, sin, rot, q, cache.k, cache.v, cache.block_table, step.token_seq,
-                                    step.token_pos, write_kv=owns_cache, n_splits=max(splits, 1), pairing=self.pairing)
-            ops.attention(q, o, cache.k, cache.v, cache.block_table, step.token_seq, step.token_pos,
-                          s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, workspace=ws.scratch(),
-                          cu_seqlens=step.cu_seqlens, max_new=step.max_new, q_counts=step.new_counts,
-                          max_len=step.max_len, n_splits=self._decode_splits(step, cache))
+            if not splits and self._fused_prefill(step, cache):
+                # A prompt step: keys and values are prepared and appended, the attention kernel
+                # prepares its queries from the projection itself.
+                if owns_cache:
+                    ops.qk_norm_rope_append(qkv, s.n_heads, s.n_kv_heads, s.head_dim, self.q_gain, self.k_gain, eps,
+                                            cos, sin, rot, None, cache.k, cache.v, cache.block_table, step.token_seq,
+                                            step.token_pos, write_kv=True, pairing=self.pairing)
+                ops.attention_prefill_fused(qkv, o, cache.k, cache.v, cache.block_table, step.token_pos, s.n_heads,
+                                            s.n_kv_heads, s.head_dim, s.scale, self.q_gain, eps, cos, sin, s.window,
+                                            step.cu_seqlens, step.new_counts)
+            else:
+                q = ws.get("attn.q", (n, self.q_dim), self.dtype)
+                ops.qk_norm_rope_append(qkv, s.n_heads, s.n_kv_heads, s.head_dim, self.q_gain, self.k_gain, eps,
+                                        cos, sin, rot, q, cache.k, cache.v, cache.block_table, step.token_seq,
+                                        step.token_pos, write_kv=owns_cache, n_splits=max(splits, 1), pairing=self.pairing)
+                ops.attention(q, o, cache.k, cache.v, cache.block_table, step.token_seq, step.token_pos,
+                              s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, workspace=ws.scratch(),
+                              cu_seqlens=step.cu_seqlens, max_new=step.max_new, q_counts=step.new_counts,
+                              max_len=step.max_len, n_splits=self._decode_splits(step, cache))
         stream(step).add_product(o, self.w_o, x_accum)
 
 

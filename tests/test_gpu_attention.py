@@ -387,6 +387,66 @@ def _long_case(length, n_new, hq, hkv, d, window, n_splits, seed):
     assert float((ref[0, 0] - vs[0][:length - n_new, 0].double().mean(0)).abs().max()) > 0.1
 
 
+# (Hq, Hkv, D, (context length after the step, new tokens) per sequence, window, norm, rotation)
+PREFILL_FUSED = [(16, 8, 128, [(300, 300)], None, True, True), (8, 2, 128, [(5, 5), (200, 130), (64, 64), (129, 1), (400, 257)], None, True, True),
+                 (8, 2, 128, [(900, 600), (70, 3)], 70, True, True), (4, 1, 64, [(130, 130), (31, 31)], None, True, False),
+                 (6, 2, 32, [(77, 50)], None, False, True), (12, 4, 96, [(200, 129), (10, 10)], 24, True, True),
+                 (6, 3, 192, [(150, 100)], None, True, True), (4, 2, 256, [(100, 64), (65, 65)], None, False, False)]
+
+
+@pytest.mark.parametrize("hq,hkv,d,seqs,window,norm,rotate", PREFILL_FUSED)
+def test_prefill_fused_prepares_its_queries(hq, hkv, d, seqs, window, norm, rotate):
+    """The prompt kernel that takes its queries from the q/k/v projection (norm, rotation and
+    rounding inside) against the two kernels it replaces, on the same projection, and against the
+    64-bit attention over the queries those prepared.  The caches must come out bit for bit the
+    same: keys and values go through the same kernel either way."""
+    dev, ks, vs, qs = _build(seqs, hq, hkv, d, torch.bfloat16, 21)
+    n = sum(m for _, m in seqs)
+    g = torch.Generator().manual_seed(22)
+    rows = hq + 2 * hkv
+    # (queries as large as the other tests': the norm brings them there, without it the projection does)
+    proj = (torch.randn(n, rows * d, generator=g) * (1.5 if norm else 1.0)).cuda()
+    q_gain = (1 + 0.3 * torch.randn(d, generator=g)).cuda() if norm else None
+    k_gain = (1 + 0.3 * torch.randn(d, generator=g)).cuda() if norm else None
+    eps = 3e-5
+    cos = sin = None
+    if rotate:
+        angle = dev["tok_pos"].float()[:, None] * (10000.0 ** (-torch.arange(d // 2, device="cuda").float() / (d // 2)))[None, :]
+        cos, sin = torch.cos(angle).contiguous(), torch.sin(angle).contiguous()
+    scale = 1.0 / math.sqrt(d)
+    ws = torch.empty(32 << 20, dtype=torch.uint8, device="cuda")
+    counts = [m for _, m in seqs]
+    # the two kernels
+    kc2, vc2 = dev["kc"].clone(), dev["vc"].clone()
+    q_dev = torch.empty(n, hq * d, dtype=torch.bfloat16, device="cuda")
+    ops.qk_norm_rope_append(proj, hq, hkv, d, q_gain, k_gain, eps, cos, sin, d if rotate else 0, q_dev, kc2, vc2,
+                            dev["table"], dev["tok_seq"], dev["tok_pos"])
+    out2 = torch.full_like(q_dev, float("nan"))
+    ops.attention(q_dev, out2, kc2, vc2, dev["table"], dev["tok_seq"], dev["tok_pos"], hq, hkv, d, scale, window,
+                  algo=MFMA, workspace=ws, cu_seqlens=dev["cu"], max_new=max(counts), q_counts=counts,
+                  max_len=max(length for length, _ in seqs))
+    # the append without queries, then the kernel that prepares them
+    ops.qk_norm_rope_append(proj, hq, hkv, d, q_gain, k_gain, eps, cos, sin, d if rotate else 0, None, dev["kc"], dev["vc"],
+                            dev["table"], dev["tok_seq"], dev["tok_pos"])
+    out = torch.full_like(q_dev, float("nan"))
+    ops.attention_prefill_fused(proj, out, dev["kc"], dev["vc"], dev["table"], dev["tok_pos"], hq, hkv, d, scale,
+                                q_gain, eps, cos, sin, window, dev["cu"], counts)
+    torch.cuda.synchronize()
+    assert torch.equal(dev["kc"], kc2) and torch.equal(dev["vc"], vc2)
+    got = out.cpu().double().reshape(n, hq, d)
+    assert float((got - out2.cpu().double().reshape(n, hq, d)).abs().max()) < 2e-2
+    # the 64-bit attention over the prepared queries and the cache's keys and values
+    table, at = dev["table"].cpu(), 0
+    kc_cpu, vc_cpu = kc2.cpu(), vc2.cpu()
+    for b, (length, m) in enumerate(seqs):
+        k = torch.stack([kc_cpu[int(table[b, p_ // PAGE]), :, p_ % PAGE] for p_ in range(length)])
+        v = torch.stack([vc_cpu[int(table[b, p_ // PAGE]), :, :, p_ % PAGE] for p_ in range(length)])
+        ref = _reference_rows(q_dev[at:at + m].cpu().reshape(m, hq, d), k, v, list(range(length - m, length)), scale, window)
+        err = float((got[at:at + m] - ref).abs().max())
+        assert err < 1.5e-2, f"sequence {b} of length {length} with {m} new tokens: error {err}"
+        at += m
+
+
 @pytest.mark.parametrize("climb", [30.0, 4.0, -30.0])
 def test_prompt_whose_scores_climb_slowly(climb):
     """The prefill kernel moves the reference of a row's exponents only when the row's maximum has
