@@ -24,6 +24,7 @@ from .residual import stream
 
 class Attention(Mixer):
     adds_only = True
+    FUSED_PREFILL_MIN_TOKENS = 1024
 
     def __init__(self, spec: AttentionSpec, ctx: BuildContext):
         if spec.n_heads % spec.n_kv_heads != 0:
@@ -96,8 +97,12 @@ class Attention(Mixer):
             self.dtype, self.spec.n_heads, self.spec.n_kv_heads, self.spec.head_dim, ops.FUSED_DECODE_PAGE, rot, self.pairing)
 
     def _fused_prefill(self, step, cache) -> bool:
+        """Whether the prompt kernel prepares its queries itself: it pays from about a thousand
+        tokens on (the preparation lengthens every attention block by some 6 us, the norm-and-rotation
+        kernel's q rows cost 8 us per thousand tokens at 32 heads of 128)."""
         rot = None if self.position is None else self.position.rot_dim
-        return (step.max_new > 1 and step.cu_seqlens is not None and self.dtype == torch.bfloat16
+        return (step.max_new > 1 and step.n_tokens >= self.FUSED_PREFILL_MIN_TOKENS
+                and step.cu_seqlens is not None and self.dtype == torch.bfloat16
                 and ops.attention_prefill_fusable(cache.k.dtype, self.spec.head_dim, cache.k.shape[2], rot, self.pairing))
 
     def takes_row_scale(self, step) -> bool:

@@ -236,6 +236,35 @@ def test_many_sequences_in_a_step(models, name, dtype, n_seqs):
     engine.cache.check()
 
 
+@pytest.mark.parametrize("name", ["B", "D", "G", "H"])
+def test_prompt_steps_whose_attention_prepares_its_queries(models, name, monkeypatch):
+    """Long prompt steps hand the attention kernel the q/k/v projection instead of prepared
+    queries.  With the length from which they do so set to two tokens, the tiny configurations
+    whose head sizes the kernel knows and whose projections come whole (64 with a window in every other layer, 96, 128) go that
+    way: whole requests, the tail token by token behind such a prompt, and batches of unequal
+    lengths, position by position against the plain implementation that rounds where the engine does."""
+    from rocml_amd.parts.attention import Attention
+    monkeypatch.setattr(Attention, "FUSED_PREFILL_MIN_TOKENS", 2)
+    path, cfg, weights = models[name]
+    engine = _engine(path, "bfloat16")
+    calls = []
+    from rocml_amd import ops
+    real = ops.attention_prefill_fused
+    monkeypatch.setattr(ops, "attention_prefill_fused", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    tol = ROUNDED_TOL_BY_NAME.get(name, ROUNDED_TOL)
+    prompts = [helpers.random_tokens(n, cfg["vocab_size"], 900 + i) for i, n in enumerate(LENGTHS[name])]
+    refs = [_rounding_oracle(cfg, weights, p) for p in prompts]
+    for p, ref in zip(prompts, refs):
+        assert helpers.per_position(helpers.run_whole(engine, p), ref) < tol, f"whole, length {len(p)}"
+        if len(p) > 8:
+            assert helpers.per_position(helpers.run_tail_by_one(engine, p, 4), ref) < tol, f"tail, length {len(p)}"
+    got = helpers.run_batch(engine, prompts, [max(1, len(p) - 3 * (j + 1)) for j, p in enumerate(prompts)])
+    for g, ref in zip(got, refs):
+        assert helpers.per_position(g, ref) < tol
+    assert calls, "no prompt step went through the kernel that prepares its queries"
+    engine.cache.check()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_short_prompt_steps_of_a_shape_seen_before_are_replayed(models, dtype):
     """A prompt step of a shape that came before (the same token counts and first positions) is
