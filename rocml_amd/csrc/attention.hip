@@ -31,22 +31,24 @@ struct AttnArgs {
     const PrefillProj* prefill_proj = nullptr;      // prompts: the projection instead of prepared queries
 };
 
-template <int D, bool FUSED, int AHEAD>
+template <int D, bool FUSED, int AHEAD, int WAVES>
 static int launch_decode_kernel(const AttnArgs& a, int n_splits, float* part_o, float* part_ml, hipStream_t stream) {
     int group = a.hq / a.hkv;
-    int lds = 4 * group * (D + 4) * (int)sizeof(float);
+    int lds = WAVES * group * (D + 4) * (int)sizeof(float);
     static int allowed = 0;
     if (lds > allowed) {
-        if (allow_lds(attn_decode_mfma_kernel<D, FUSED, AHEAD>, lds)) return 1;
+        if (allow_lds(attn_decode_mfma_kernel<D, FUSED, AHEAD, WAVES>, lds)) return 1;
         allowed = lds;
     }
     dim3 grid(n_splits, a.hkv, a.n_tokens);
-    attn_decode_mfma_kernel<D, FUSED, AHEAD><<<grid, AM_THREADS, lds, stream>>>(
+    attn_decode_mfma_kernel<D, FUSED, AHEAD, WAVES><<<grid, 64 * WAVES, lds, stream>>>(
         a.q, a.out, const_cast<bf16_t*>(a.kcache), const_cast<bf16_t*>(a.vcache), a.block_table, a.bt_width,
         a.token_seq, a.token_pos, a.hq, a.hkv, a.scale * LOG2E, a.window, n_splits, part_o, part_ml,
         FUSED ? *a.proj : DecodeProj{});
     return 0;
 }
+
+constexpr int WIDE_BLOCK_MIN_PIECES = 8;         // of a block: more than two a wave of four
 
 template <int D, bool FUSED>
 static int launch_decode(const AttnArgs& a, hipStream_t stream) {
@@ -69,13 +71,21 @@ static int launch_decode(const AttnArgs& a, hipStream_t stream) {
     // do when the chip holds at most one block a CU (a long loop then gains from it what a second
     // block would bring).  The choice follows the launch's shape, not the lengths, as the number of
     // splits does.
+    // Eight waves a block where the chip holds at most one block a CU and a block of four waves
+    // could give a wave more pieces than two trips bring (the pages the block table has room for,
+    // two pieces each, over the splits and the waves: the launch's shape again, not the lengths).
     int rc;
-    if constexpr (D <= 128)
-        rc = n_splits >= 4 || (long long)a.n_tokens * a.hkv * n_splits <= cu_count()
-                 ? launch_decode_kernel<D, FUSED, 2>(a, n_splits, part_o, part_ml, stream)
-                 : launch_decode_kernel<D, FUSED, 1>(a, n_splits, part_o, part_ml, stream);
-    else
-        rc = launch_decode_kernel<D, FUSED, 1>(a, n_splits, part_o, part_ml, stream);
+    if constexpr (D <= 128) {
+        bool one_a_cu = (long long)a.n_tokens * a.hkv * n_splits <= cu_count();
+        long long pieces = 2ll * ((a.bt_width + n_splits - 1) / n_splits);
+        if (one_a_cu && pieces > WIDE_BLOCK_MIN_PIECES)
+            rc = launch_decode_kernel<D, FUSED, 2, 8>(a, n_splits, part_o, part_ml, stream);
+        else
+            rc = n_splits >= 4 || one_a_cu ? launch_decode_kernel<D, FUSED, 2, 4>(a, n_splits, part_o, part_ml, stream)
+                                           : launch_decode_kernel<D, FUSED, 1, 4>(a, n_splits, part_o, part_ml, stream);
+    } else {
+        rc = launch_decode_kernel<D, FUSED, 1, 4>(a, n_splits, part_o, part_ml, stream);
+    }
     if (rc) return rc;
     if (n_splits > 1)
         // whole waves: the kernel's reductions exchange values between all 64 lanes

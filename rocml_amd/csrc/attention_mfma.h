@@ -54,7 +54,7 @@ struct DecodeProj {
     const float* row_ssq; int row_parts; float row_eps; float row_inv_width;
 };
 
-// grid (n_splits, Hkv, tokens), 4 waves; the block's pages are cut into 32-key pieces that the
+// grid (n_splits, Hkv, tokens), 4 or 8 waves; the block's pages are cut into 32-key pieces that the
 // waves take in turn; all query heads of the kv head ride in the 16 columns of the MFMA.
 //
 // FUSED: the kernel takes the projection's output instead of q and a finished cache: every block
@@ -63,8 +63,10 @@ struct DecodeProj {
 // and the new value into the cache and multiplies them as one more piece, from LDS: the loads
 // from the cache may or may not see a row that is written in the same launch, so the cached
 // keys end before it.  A page belongs to one split, so no other block reads that row.
-template <int D, bool FUSED, int AHEAD>
-__global__ void __launch_bounds__(AM_THREADS)
+// WAVES: 4, or 8 for launches of at most one block a CU whose blocks have many pieces: a wave
+// then has half as many, and the pieces of a block travel in half as many trips.
+template <int D, bool FUSED, int AHEAD, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES)
 attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                         bf16_t* kcache, bf16_t* vcache,
                         const int* __restrict__ block_table, int bt_width,
@@ -73,8 +75,9 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                         float* __restrict__ part_o, float* __restrict__ part_ml, DecodeProj pj) {
     constexpr int KD = D / 32;      // MFMA steps along D for the scores
     constexpr int DT = D / 16;      // 16-row tiles of the output
-    extern __shared__ float sm_o[];                 // [4 waves][group][D + 4]
-    __shared__ float sm_m[4][16], sm_l[4][16];
+    constexpr int THREADS = 64 * WAVES;
+    extern __shared__ float sm_o[];                 // [WAVES][group][D + 4]
+    __shared__ float sm_m[WAVES][16], sm_l[WAVES][16];
     int split = blockIdx.x, kvh = blockIdx.y, t = blockIdx.z;
     int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     int g = lane >> 4, col = lane & 15;
@@ -127,7 +130,7 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     // The wave's first pieces are requested before the queries: their keys and values travel
     // together with them.
     if (wave < n_pieces) request_piece(wave, kbuf[0], vbuf[0]);
-    if (AHEAD == 2 && wave + 4 < n_pieces) request_piece(wave + 4, kbuf[AHEAD - 1], vbuf[AHEAD - 1]);
+    if (AHEAD == 2 && wave + WAVES < n_pieces) request_piece(wave + WAVES, kbuf[AHEAD - 1], vbuf[AHEAD - 1]);
     // Q^T operand: column = head of the group (zero beyond it), 8 values of D per lane and step.
     bf16x8_t qf[KD];
     bool owner = false;      // this block appends the new key and value
@@ -147,7 +150,7 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         // takes a row at a time, a lane the values lane, lane + 64, ...; two rows per wave are
         // loaded together, so a group of four heads with key and value is one trip to memory.
         constexpr int J = D / 64;
-        __shared__ float sm_f[AM_THREADS / 64][2][D];                        // a row before its rotation
+        __shared__ float sm_f[WAVES][2][D];                        // a row before its rotation
         __shared__ __attribute__((aligned(16))) bf16_t sm_q[16 * D];        // [head of the group][D]
         __shared__ __attribute__((aligned(16))) bf16_t sm_knew[D];
         __shared__ __attribute__((aligned(16))) bf16_t sm_vnew[D];
@@ -169,13 +172,13 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
             }
             row_scale = 1.0f / sqrtf(wave_sum(ss) * pj.row_inv_width + pj.row_eps);
         }
-        for (int base = 0; base < n_rows; base += 2 * (AM_THREADS / 64)) {
+        for (int base = 0; base < n_rows; base += 2 * WAVES) {
             int r[2];
             const float* src[2];
             float raw[2][J][4];
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
-                r[i] = base + i * (AM_THREADS / 64) + wave;
+                r[i] = base + i * WAVES + wave;
                 int prow = r[i] < group ? kvh * group + r[i] : (r[i] == group ? hq + kvh : hq + hkv + kvh);
                 src[i] = tok + (size_t)(r[i] < n_rows ? prow : 0) * D + lane;
 #pragma unroll
@@ -308,18 +311,18 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     // (FUSED: the new key is not yet in the cache where a block reads it; it comes last, from LDS)
     int cached = (FUSED && owner) ? new_pos : len;
     auto first_key = [&](int piece) { return (first_page + split + (piece >> 1) * n_splits) * AM_PAGE + (piece & 1) * 32; };
-    for (int piece = wave; piece < n_pieces; piece += 4 * AHEAD) {
+    for (int piece = wave; piece < n_pieces; piece += WAVES * AHEAD) {
         multiply_piece(first_key(piece), lo, cached, kbuf[0], vbuf[0]);
-        if (piece + 4 * AHEAD < n_pieces) request_piece(piece + 4 * AHEAD, kbuf[0], vbuf[0]);
-        if (AHEAD == 2 && piece + 4 < n_pieces) {
-            multiply_piece(first_key(piece + 4), lo, cached, kbuf[AHEAD - 1], vbuf[AHEAD - 1]);
-            if (piece + 12 < n_pieces) request_piece(piece + 12, kbuf[AHEAD - 1], vbuf[AHEAD - 1]);
+        if (piece + WAVES * AHEAD < n_pieces) request_piece(piece + WAVES * AHEAD, kbuf[0], vbuf[0]);
+        if (AHEAD == 2 && piece + WAVES < n_pieces) {
+            multiply_piece(first_key(piece + WAVES), lo, cached, kbuf[AHEAD - 1], vbuf[AHEAD - 1]);
+            if (piece + 3 * WAVES < n_pieces) request_piece(piece + 3 * WAVES, kbuf[AHEAD - 1], vbuf[AHEAD - 1]);
         }
     }
     if constexpr (FUSED) {
         // The step's own key and value as a piece of their own, row 0 of score tile 0, in the
         // wave whose turn would be next.
-        if (owner && wave == (n_pieces & 3)) {
+        if (owner && wave == n_pieces % WAVES) {
             bool krow = col == 0, vrow = g == 0;
 #pragma unroll
             for (int u = 0; u < 2; ++u)
@@ -335,7 +338,7 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
             multiply_piece(new_pos, new_pos, new_pos + 1, kbuf[0], vbuf[0]);
         }
     }
-    // merge the four waves in wave order; element i of o[dt] is d = 16 dt + 4g + i, column = head.
+    // merge the waves in wave order; element i of o[dt] is d = 16 dt + 4g + i, column = head.
     if (col < group) {
         float* mine = sm_o + ((size_t)wave * group + col) * (D + 4);
 #pragma unroll
@@ -348,12 +351,14 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         sm_l[wave][col] = l;
     }
     __syncthreads();
-    for (int idx = tid; idx < group * D; idx += AM_THREADS) {
+    for (int idx = tid; idx < group * D; idx += THREADS) {
         int head = idx / D, d = idx - head * D;
-        float mm = fmaxf(fmaxf(sm_m[0][head], sm_m[1][head]), fmaxf(sm_m[2][head], sm_m[3][head]));
+        float mm = sm_m[0][head];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) mm = fmaxf(mm, sm_m[w][head]);
         float ll = 0.f, acc = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
+        for (int w = 0; w < WAVES; ++w) {
             float wgt = sm_m[w][head] == -INFINITY ? 0.f : fast_exp2(sm_m[w][head] - mm);
             ll += sm_l[w][head] * wgt;
             acc += sm_o[((size_t)w * group + head) * (D + 4) + d] * wgt;
