@@ -499,11 +499,12 @@ def attention_prefill_fused(qkv: torch.Tensor, out: torch.Tensor, k_cache: torch
                             block_table: torch.Tensor, token_pos: torch.Tensor, n_heads: int, n_kv_heads: int,
                             head_dim: int, scale: float, q_gain: Optional[torch.Tensor], eps: float,
                             cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], window: Optional[int],
-                            cu_seqlens: torch.Tensor, q_counts: Sequence[int]) -> None:
+                            cu_seqlens: torch.Tensor, q_counts: Sequence[int], max_len: int = 0) -> None:
     """A prompt step's attention with the queries taken from the q/k/v projection ``qkv`` (float32
     ``[tokens, ld]``, complete sums, a token's q heads first): per-head norm, rotation and rounding
     of the queries happen in the attention kernel.  The new tokens' keys and values are in the
-    cache already (``qk_norm_rope_append`` without a q output puts them there)."""
+    cache already (``qk_norm_rope_append`` without a q output puts them there).  ``max_len``
+    (the longest context) is what ``--profile`` prices the call with; the kernel does not need it."""
     _dev(qkv, out, k_cache, v_cache, block_table, token_pos, q_gain, cos, sin, cu_seqlens)
     _want(qkv, torch.float32, "projection output")
     if qkv.dim() != 2:

@@ -162,7 +162,7 @@ class Attention(Mixer):
                                             step.token_pos, write_kv=True, pairing=self.pairing)
                 ops.attention_prefill_fused(qkv, o, cache.k, cache.v, cache.block_table, step.token_pos, s.n_heads,
                                             s.n_kv_heads, s.head_dim, s.scale, self.q_gain, eps, cos, sin, s.window,
-                                            step.cu_seqlens, step.new_counts)
+                                            step.cu_seqlens, step.new_counts, max_len=step.max_len)
             else:
                 q = ws.get("attn.q", (n, self.q_dim), self.dtype)
                 ops.qk_norm_rope_append(qkv, s.n_heads, s.n_kv_heads, s.head_dim, self.q_gain, self.k_gain, eps,

@@ -64,6 +64,15 @@ def _fused_attention_cost(qkv, out, k_cache, v_cache, block_table, token_seq, to
     return _nbytes(qkv, out) + kv, 4 * n_heads * head_dim * n_seqs * max_len
 
 
+def _prefill_fused_cost(qkv, out, k_cache, v_cache, block_table, token_pos, n_heads, n_kv_heads, head_dim,
+                        scale, q_gain, eps, cos, sin, window, cu_seqlens, q_counts, max_len=0) -> Tuple[int, int]:
+    n_tokens, n_seqs, max_new = qkv.shape[0], len(q_counts), max(q_counts)
+    kv = 2 * n_seqs * max_len * n_kv_heads * head_dim * k_cache.element_size()
+    keys_per_query = max(1, max_len - max_new // 2)                                   # causal: half of the new part
+    read_q = n_tokens * n_heads * head_dim * qkv.element_size()                       # the q columns of the projection
+    return read_q + _nbytes(out, cos, sin) + kv, 4 * n_heads * head_dim * n_tokens * keys_per_query
+
+
 def _tensor_args_cost(skip: Tuple[int, ...] = (), flops_per_byte: float = 0.0) -> Callable:
     def cost(*a, **kw) -> Tuple[int, int]:
         tensors = [t for i, t in enumerate(a) if i not in skip] + list(kw.values())
@@ -79,6 +88,7 @@ _COSTS: Dict[str, Tuple[str, Callable]] = {
         _nbytes(x, w, resid, resid, gain, xg, ssq), 2 * x.shape[0] * w.shape[0] * x.shape[1])),
     "attention": ("attention", _attention_cost),
     "attention_decode_fused": ("attention (norm, rotation, append)", _fused_attention_cost),
+    "attention_prefill_fused": ("attention (query norm, rotation)", _prefill_fused_cost),
     "qk_norm_rope_append": ("q/k norm, rotation, append", _tensor_args_cost(skip=(11, 12))),   # not the whole cache
     "rmsnorm": ("rmsnorm", _tensor_args_cost(flops_per_byte=0.5)),
     "swiglu": ("swiglu", _tensor_args_cost(flops_per_byte=0.5)),
